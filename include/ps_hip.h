@@ -55,12 +55,15 @@ enum ps_dtype {
     PS_Q6_K = 14,
     PS_Q8_K = 15,
     PS_I32  = 26,
+    PS_BF16 = 30, /* dense matrices of the layer-list models (ps_hip_dense_upload) */
 };
 
 typedef struct ps_hip_ctx ps_hip_ctx;
 typedef struct ps_weight ps_weight;   /* device-resident quantized weight matrix [K, N] */
 typedef struct ps_hip_model ps_hip_model;
 typedef struct ps_hip_graph ps_hip_graph;
+typedef struct ps_dense ps_dense;         /* device-resident dense matrix [N, K], bfloat16 or float32 */
+typedef struct ps_hip_seq ps_hip_seq;     /* a layer-list model with its pool of sequence states */
 
 typedef struct {
     int32_t dtype;
@@ -290,6 +293,95 @@ int ps_hip_debug_f16_gemm(ps_hip_ctx *ctx, int M, int64_t N, int64_t K, int reps
  * (the fused launch contains the one-launch attention's exchange, its time-out is the same flag and the same fallback).
  * The environment variable PS_HIP_MODE_OR is OR-ed into every mode (A/B runs of unmodified drivers). */
 int ps_hip_model_set_mode(ps_hip_model *m, int mode);
+
+
+/* ------------------------------------------------------------------ layer-list models
+ * Models that are a LIST of layers, each one token mixer of some kind plus an optional feed-forward, with dense
+ * (unquantized) matrices: recurrent mixers whose memory is a fixed-size state, and windowed latent attention whose
+ * memory is a ring of compressed keys.  Every size and constant comes in through the descriptors; the mechanisms
+ * (csrc/k_seqmix.hip, k_latent.hip, k_dense.hip) take them as launch parameters.
+ *
+ * Numerics: matrix products run on bfloat16 operands with fp32 accumulation (compute == 0) or entirely in fp32
+ * (compute == 1, no reduced-precision matrix mode); everything else -- the residual stream, norms, positions and angles,
+ * scores and soft-max, decays, gates of a recurrence and the recurrent state -- is fp32 in both. */
+enum ps_mixer_kind {
+    PS_MIX_WKV    = 1, /* per-channel decayed outer-product state, token-shift mixes, bonus for the current token */
+    PS_MIX_DELTA  = 2, /* gated delta rule: per-head scalar decay, write strength beta, short convolutions on q / k / v */
+    PS_MIX_LATENT = 3, /* attention over a low-rank latent + one shared rotated key part, sliding window */
+};
+enum ps_ff_kind { PS_FF_NONE = 0, PS_FF_DENSE_XIELU = 1 };
+
+/* Dense matrix [N rows = outputs][K = inputs], row-major, applied as W x.  host_bf16: N*K bfloat16 bit patterns.
+ * as_f32 != 0 widens it to fp32 on the device (the fp32 compute mode). */
+int ps_hip_dense_upload(ps_hip_ctx *ctx, const uint16_t *host_bf16, int64_t N, int64_t K, int as_f32, ps_dense **out);
+void ps_hip_dense_free(ps_hip_ctx *ctx, ps_dense *w);
+/* out[T][N] = alpha * (x[T][K] . W^T), device fp32 in and out (tests, micro-benchmarks; the model uses the same launchers) */
+int ps_hip_dense_matmul(ps_hip_ctx *ctx, const ps_dense *w, const float *x_dev, int T, float *out_dev, float alpha);
+
+typedef struct {
+    int32_t kind;     /* ps_mixer_kind */
+    int32_t heads, kv_heads, dim, vdim; /* q/k size per head, value size per head (wkv: vdim == dim) */
+    int32_t conv_taps;                  /* delta: taps of the short convolutions on q / k / v */
+    int32_t decay_rank;                 /* wkv: inner size of the decay's two-matrix projection */
+    int32_t q_rank, kv_rank, rot_dim;   /* latent: ranks of the query / key-value latents, size of the rotated part */
+    int32_t rot_dims;                   /* latent: how many numbers of the rotated part turn (pairs (i, i + rot_dims / 2)); the rest pass unchanged */
+    int32_t window;                     /* latent: a position sees itself and the window - 1 before it */
+    float rot_base, scale;              /* latent: rotary base (angle of pair i at position p: p * base^(-2 i / rot_dims)), score scale */
+    int32_t ff_kind, ff;                /* feed-forward kind and inner size (PS_FF_NONE: the layer has none) */
+    float ff_act_p, ff_act_q;           /* xIELU: the two raw numbers (softplus is applied by the library) */
+    /* vectors: device fp32.  norm1 / norm2 / norm1b / norm2b [width]; canon1 / canon2 [width][canon_taps] */
+    const float *norm1, *norm2, *norm1b, *norm2b, *canon1, *canon2;
+    /* matrices (NULL where the kind has none):
+     *   wkv:    in_r, in_k, in_v, in_g [heads*dim, width], decay1 [decay_rank, width], decay2 [heads*dim, decay_rank], out
+     *   delta:  in_cat = rows of q | k | v | g | b | a  ([2*kv_heads*dim + 2*heads*vdim + 2*heads, width]), out
+     *   latent: in_cat = rows of dq | dkv ([q_rank + kv_rank + rot_dim, width]), uq [heads*(dim+rot_dim), q_rank],
+     *           ukv = rows of uk | uv ([heads*dim + heads*vdim, kv_rank]), out */
+    const ps_dense *in_r, *in_k, *in_v, *in_g, *decay1, *decay2, *in_cat, *uq, *ukv, *out, *ff_up, *ff_down;
+    /* wkv: mu [5][width] in the order r, k, v, g, w; decay0 [heads*dim]; bonus [heads*dim]; onorm [heads*dim]
+     * delta: conv [2*kv_heads*dim + heads*vdim][conv_taps] (rows q | k | v); a_log, dt_bias [heads]; onorm [vdim]
+     * latent: qnorm [q_rank], kvnorm [kv_rank] */
+    const float *mu, *decay0, *bonus, *onorm, *conv, *a_log, *dt_bias, *qnorm, *kvnorm;
+} ps_seq_layer;
+
+typedef struct {
+    int32_t n_layers, width, vocab, canon_taps;
+    int32_t max_batch;   /* most tokens one launch sequence takes; longer inputs are cut into portions of this size */
+    int32_t n_slots;     /* sequence states held at once */
+    int32_t compute;     /* 0: bfloat16 matrix products, 1: fp32 */
+    float norm_eps, norm_offset /* weight applied as (offset + w) */, logit_scale;
+    const ps_dense *embed, *head; /* [vocab, width] both */
+    const float *final_norm;
+    const ps_seq_layer *layers;
+} ps_seq_desc;
+
+int ps_hip_seq_create(ps_hip_ctx *ctx, const ps_seq_desc *desc, ps_hip_seq **out);
+void ps_hip_seq_destroy(ps_hip_seq *m);
+/* State manager: a slot holds everything a sequence carries from token to token (convolution tails, token-shift rows,
+ * recurrent states, the latent ring) and its position.  acquire hands out a zeroed slot at position 0 (-1 in *slot and a
+ * non-zero return when none is free); release gives it back for reuse. */
+int ps_hip_seq_acquire(ps_hip_seq *m, int *slot);
+int ps_hip_seq_release(ps_hip_seq *m, int slot);
+int64_t ps_hip_seq_position(const ps_hip_seq *m, int slot);
+size_t ps_hip_seq_slot_bytes(const ps_hip_seq *m);
+/* The step function: the next n tokens of the sequence in `slot` (HOST ids), from the state earlier steps left.
+ * want: n_want indices into these tokens (HOST, may be NULL) whose logits are written to logits_host [n_want][vocab]
+ * and whose arg-max ids to argmax_host (either may be NULL). */
+int ps_hip_seq_forward(ps_hip_seq *m, int slot, const int32_t *tokens, int n, const int32_t *want, int n_want,
+                       float *logits_host, int32_t *argmax_host);
+/* Greedy single-token steps: feeds `token`, then its own arg-max, `steps` times (captured launch sequence, no host round trip
+ * per token).  out_ids HOST int32[steps]. */
+int ps_hip_seq_decode_greedy(ps_hip_seq *m, int slot, int32_t token, int steps, int32_t *out_ids);
+/* diagnostics: with buf != NULL (device, [n_layers][max_batch][width] fp32) every forward of at most max_batch tokens leaves
+ * the residual stream after each layer there */
+int ps_hip_seq_debug_layers(ps_hip_seq *m, float *buf_dev);
+/* bit 0: 1 = eager launches for the single-token step (default: hipGraph replay); bit 1: 1 = the unfused reference kernels
+ * wherever a faster form exists (per-key attention, tiled mat-mul for single tokens) -- same results up to rounding */
+int ps_hip_seq_set_mode(ps_hip_seq *m, int mode);
+uint64_t ps_hip_seq_weight_bytes_per_token(const ps_hip_seq *m);
+/* Measurement helper: one kernel family of the step function replayed `reps` times on the model's own buffers between
+ * HIP events -> microseconds per launch and the bytes / flops it moves (bench.py's per-kernel roofline).
+ * which: 0 feed-forward up mat-vec (single token), 1 the same for T tokens, 2 wkv scan, 3 delta scan, 4 latent attention */
+int ps_hip_seq_bench_kernel(ps_hip_seq *m, int which, int T, int reps, double *us_per_launch, double *bytes, double *flops);
 
 #ifdef __cplusplus
 }

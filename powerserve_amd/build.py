@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(HERE, "build")
-SOURCES = ["api.hip", "model.hip", "k_quant.hip", "k_gemv.hip", "k_gemv4.hip", "k_qkvattn.hip", "k_gemvb.hip", "k_gemvk.hip", "k_gemm4k.hip", "k_gemv6.hip", "k_ops.hip", "k_attn.hip", "perf16.hip"]
+SOURCES = ["ctx.hip", "api.hip", "model.hip", "k_quant.hip", "k_gemv.hip", "k_gemv4.hip", "k_qkvattn.hip", "k_gemvb.hip", "k_gemvk.hip", "k_gemm4k.hip", "k_gemv6.hip", "k_ops.hip", "k_attn.hip", "perf16.hip", "seqmodel.hip", "k_dense.hip", "k_seqmix.hip", "k_latent.hip"]
 # -ffp-contract=off: the parity contract needs every fp32 op to round where the reference's C source rounds;
 # fused multiply-adds are written explicitly (__fmaf_rn) where the reference uses FMA intrinsics.
 # -fno-slp-vectorize (NOSLP files only): hipcc's SLP vectoriser packs adjacent scalar fp32 operations into v_pk_fma_f32 / v_pk_mul_f32 / v_pk_add_f32.  On
@@ -22,6 +22,11 @@ SOURCES = ["api.hip", "model.hip", "k_quant.hip", "k_gemv.hip", "k_gemv4.hip", "
 # exact compile configuration that has passed the full GPU suite and all bench configurations.)
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-Wno-unused-result",
          "-I" + os.path.join(HERE, "..", "include")]
+# The layer-list models (dense bf16 / fp32 matrices; include/ps_hip.h): their sources plus the context make a library of their own,
+# lib/libps_hip_seq.so, so that a checkout that only serves such a model compiles four files and not the quantized path's kernels.
+SEQ_SOURCES = ["ctx.hip", "seqmodel.hip", "k_dense.hip", "k_seqmix.hip", "k_latent.hip"]
+# packed fp32 instructions are left to no one: these files are ordinary float code and are compiled without the feature
+SEQ_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 NOSLP = {"k_gemv4.hip", "k_qkvattn.hip", "k_gemvb.hip", "k_attn.hip", "k_gemm4k.hip"}  # k_gemm4k.hip (round 5): gate/up chunk launch of a 512-column sequence 384.2 -> 369-371 us, same bits (profiles/r05_g4k2_variants.txt, the "v2 0" lines vs profiles/r05_g4k_item_order.txt)  # (k_gemvb.hip: the Q4_0 / Q8_0 mat-vec, Llama-3.2-1B 1494 -> 1525 tok/s)
 
 
@@ -52,6 +57,39 @@ CONTRACT_SOURCES = {"api.hip", "k_ops.hip", "k_attn.hip", "k_gemm4k.hip", "k_gem
 TIMELINE_SOURCES = {"api.hip", "k_gemv4.hip", "k_qkvattn.hip", "k_attn.hip", "k_gemm4k.hip"}
 
 
+def _compile_cmd(hipcc: str, s: str, src: str, obj: str) -> list:
+    return [hipcc, *FLAGS, *(["-fno-slp-vectorize"] if s in NOSLP else []), *(SEQ_FLAGS if s in SEQ_SOURCES and s != "ctx.hip" else []), "-c", src, "-o", obj]
+
+
+def build_seq(force: bool = False, verbose: bool = True) -> str:
+    """lib/libps_hip_seq.so: the context and the layer-list models only (the objects are shared with the full library's build)."""
+    os.makedirs(LIBDIR, exist_ok=True)
+    os.makedirs(OBJDIR, exist_ok=True)
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    objs, jobs = [], []
+    for s in SEQ_SOURCES:
+        src, obj = os.path.join(CSRC, s), os.path.join(OBJDIR, s.replace(".hip", ".o"))
+        objs.append(obj)
+        cmd = _compile_cmd(hipcc, s, src, obj)
+        if force or _newer(src, obj) or _cmd_changed(obj, cmd):
+            jobs.append(cmd)
+
+    def run(cmd):
+        if verbose:
+            print("[build]", os.path.basename(cmd[-1]), flush=True)
+        subprocess.run(cmd, check=True)
+        open(cmd[-1] + ".cmd", "w").write(" ".join(cmd))
+
+    with ThreadPoolExecutor(max_workers=8) as ex:
+        list(ex.map(run, jobs))
+    so = os.path.join(LIBDIR, "libps_hip_seq.so")
+    if jobs or not os.path.exists(so):
+        tmp = so + ".%d.tmp" % os.getpid()
+        subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs], check=True)
+        os.replace(tmp, so)
+    return so
+
+
 def build(force: bool = False, verbose: bool = True, contract: bool = True, timeline: bool = False) -> str:
     os.makedirs(LIBDIR, exist_ok=True)
     os.makedirs(OBJDIR, exist_ok=True)
@@ -60,7 +98,7 @@ def build(force: bool = False, verbose: bool = True, contract: bool = True, time
     for s in SOURCES:
         src, obj = os.path.join(CSRC, s), os.path.join(OBJDIR, s.replace(".hip", ".o"))
         objs.append(obj)
-        cmd = [hipcc, *FLAGS, *(["-fno-slp-vectorize"] if s in NOSLP else []), "-c", src, "-o", obj]
+        cmd = _compile_cmd(hipcc, s, src, obj)
         if force or _newer(src, obj) or _cmd_changed(obj, cmd):
             jobs.append(cmd)
         if contract and s in CONTRACT_SOURCES:
@@ -124,4 +162,7 @@ def build_host(force: bool = False, verbose: bool = True) -> str:
 
 
 if __name__ == "__main__":
-    print(build(force="--force" in sys.argv, timeline="--timeline" in sys.argv))
+    if "--seq" in sys.argv:
+        print(build_seq(force="--force" in sys.argv))
+    else:
+        print(build(force="--force" in sys.argv, timeline="--timeline" in sys.argv))

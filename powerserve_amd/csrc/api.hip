@@ -49,154 +49,10 @@ void ps_rope_table_host(const ps_rope_params *rp, int64_t ne0, const int32_t *po
 static inline bool is_quant(int t) { return t == PS_Q4_0 || t == PS_Q8_0 || t == PS_Q4_K || t == PS_Q5_K || t == PS_Q6_K; }
 static inline bool is_row_wave(int t) { return t == PS_Q5_K || t == PS_Q6_K; } // one wave per weight row (k_gemv6.hip)
 
-// ------------------------------------------------------------------ device allocations (ps_internal.h)
-namespace {
-struct GuardRec { void *va; size_t reserved, mapped; hipMemGenericAllocationHandle_t h; };
-std::mutex g_guard_mu;
-std::unordered_map<void *, GuardRec> g_guard;
-int guard_align() { static const int a = getenv("PS_HIP_GUARD") ? atoi(getenv("PS_HIP_GUARD")) : 0; return a; } // 0: off; 1: on, hipMalloc's 256-byte alignment kept; 16 / 64 / ...: that alignment
-bool guard_on() { return guard_align() != 0; }
-} // namespace
-hipError_t ps_dev_malloc(void **p, size_t bytes) {
-    if (!guard_on()) return hipMalloc(p, bytes);
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return e;
-    hipMemAllocationProp prop = {};
-    prop.type = hipMemAllocationTypePinned;
-    prop.location.type = hipMemLocationTypeDevice;
-    prop.location.id = dev;
-    size_t gran = 0;
-    if ((e = hipMemGetAllocationGranularity(&gran, &prop, hipMemAllocationGranularityMinimum)) != hipSuccess) return e;
-    const size_t al = guard_align() >= 16 ? (size_t)guard_align() : 256;
-    const size_t user = (bytes + al - 1) / al * al, mapped = (user + gran - 1) / gran * gran, reserved = mapped + gran; // (the last granule stays unmapped)
-    GuardRec r{nullptr, reserved, mapped, {}};
-    if ((e = hipMemAddressReserve(&r.va, reserved, gran, nullptr, 0)) != hipSuccess) return e;
-    if ((e = hipMemCreate(&r.h, mapped, &prop, 0)) != hipSuccess) { (void)hipMemAddressFree(r.va, reserved); return e; }
-    if ((e = hipMemMap(r.va, mapped, 0, r.h, 0)) != hipSuccess) { (void)hipMemRelease(r.h); (void)hipMemAddressFree(r.va, reserved); return e; }
-    hipMemAccessDesc acc = {};
-    acc.location = prop.location;
-    acc.flags = hipMemAccessFlagsProtReadWrite;
-    if ((e = hipMemSetAccess(r.va, mapped, &acc, 1)) != hipSuccess) { (void)hipMemUnmap(r.va, mapped); (void)hipMemRelease(r.h); (void)hipMemAddressFree(r.va, reserved); return e; }
-    *p = (char *)r.va + (mapped - user);
-    std::lock_guard<std::mutex> lk(g_guard_mu);
-    g_guard[*p] = r;
-    return hipSuccess;
-}
-hipError_t ps_dev_free(void *p) {
-    if (!p) return hipSuccess;
-    if (!guard_on()) return hipFree(p);
-    GuardRec r;
-    {
-        std::lock_guard<std::mutex> lk(g_guard_mu);
-        auto it = g_guard.find(p);
-        if (it == g_guard.end()) return hipFree(p);
-        r = it->second;
-        g_guard.erase(it);
-    }
-    // the range is never handed back: with hipMemUnmap / hipMemRelease / hipMemAddressFree behind every free, later allocations of the same process read
-    // wrong data now and then (ops tests failed at random under recycling and pass without it); a debugging run can afford the memory
-    return hipSuccess;
-}
-
 
 extern "C" {
 
-int ps_hip_abi_version(void) { return PS_HIP_ABI_VERSION; }
 int ps_hip_build_contract(void) { return PS_CONTRACT_ON ? 1 : 0; }
-
-int ps_hip_device_count(void) {
-    int n = 0;
-    if (hipGetDeviceCount(&n) != hipSuccess) return 0;
-    return n;
-}
-
-
-int ps_hip_create(int device, ps_hip_ctx **out) {
-    *out = nullptr;
-    int n = 0;
-    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0 || device >= n) return 1;
-    if (hipSetDevice(device) != hipSuccess) return 1;
-    auto c    = new ps_hip_ctx();
-    c->device = device;
-    hipDeviceProp_t prop;
-    if (hipGetDeviceProperties(&prop, device) == hipSuccess) c->n_cu = prop.multiProcessorCount;
-    if (hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking) != hipSuccess) { delete c; return 1; }
-    *out = c;
-    return 0;
-}
-
-void ps_hip_destroy(ps_hip_ctx *c) {
-    if (!c) return;
-    (void)hipSetDevice(c->device);
-    (void)hipStreamSynchronize(c->stream);
-    if (c->act_buf) (void)ps_dev_free(c->act_buf);
-    if (c->i32_buf) (void)ps_dev_free(c->i32_buf);
-    if (c->u8_buf) (void)ps_dev_free(c->u8_buf);
-    if (c->rope_buf) (void)ps_dev_free(c->rope_buf);
-    (void)hipStreamDestroy(c->stream);
-    delete c;
-}
-
-const char *ps_hip_last_error(const ps_hip_ctx *c) { return c ? c->err.c_str() : "no context"; }
-
-int ps_hip_device_name(const ps_hip_ctx *c, char *buf, size_t cap) {
-    hipDeviceProp_t prop;
-    if (hipGetDeviceProperties(&prop, c->device) != hipSuccess) return 1;
-    snprintf(buf, cap, "%s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
-    return 0;
-}
-
-int ps_hip_malloc(ps_hip_ctx *c, size_t bytes, void **dptr) {
-    PS_CHECK(c, hipSetDevice(c->device));
-    PS_CHECK(c, ps_dev_malloc(dptr, bytes ? bytes : 16));
-    return 0;
-}
-int ps_hip_free(ps_hip_ctx *c, void *dptr) {
-    PS_CHECK(c, hipStreamSynchronize(c->stream));
-    PS_CHECK(c, ps_dev_free(dptr));
-    return 0;
-}
-int ps_hip_memcpy_h2d(ps_hip_ctx *c, void *dst, const void *src, size_t bytes) {
-    PS_CHECK(c, hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, c->stream));
-    PS_CHECK(c, hipStreamSynchronize(c->stream));
-    return 0;
-}
-int ps_hip_memcpy_d2h(ps_hip_ctx *c, void *dst, const void *src, size_t bytes) {
-    PS_CHECK(c, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, c->stream));
-    PS_CHECK(c, hipStreamSynchronize(c->stream));
-    return 0;
-}
-int ps_hip_memset(ps_hip_ctx *c, void *dst, int value, size_t bytes) {
-    PS_CHECK(c, hipMemsetAsync(dst, value, bytes, c->stream));
-    return 0;
-}
-int ps_hip_sync(ps_hip_ctx *c) {
-    PS_CHECK(c, hipStreamSynchronize(c->stream));
-    PS_CHECK(c, hipGetLastError());
-    return 0;
-}
-void *ps_hip_stream(ps_hip_ctx *c) { return (void *)c->stream; }
-
-int ps_hip_event_create(ps_hip_ctx *c, void **ev) {
-    hipEvent_t e;
-    PS_CHECK(c, hipEventCreate(&e));
-    *ev = (void *)e;
-    return 0;
-}
-int ps_hip_event_record(ps_hip_ctx *c, void *ev) {
-    PS_CHECK(c, hipEventRecord((hipEvent_t)ev, c->stream));
-    return 0;
-}
-int ps_hip_event_elapsed_ms(ps_hip_ctx *c, void *a, void *b, float *ms) {
-    PS_CHECK(c, hipEventSynchronize((hipEvent_t)b));
-    PS_CHECK(c, hipEventElapsedTime(ms, (hipEvent_t)a, (hipEvent_t)b));
-    return 0;
-}
-int ps_hip_event_destroy(ps_hip_ctx *c, void *ev) {
-    PS_CHECK(c, hipEventDestroy((hipEvent_t)ev));
-    return 0;
-}
 
 // ------------------------------------------------------------------ type helpers (ggml.c:681-1015)
 size_t ps_hip_row_size(int t, int64_t k) {

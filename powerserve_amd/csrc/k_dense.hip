@@ -1,0 +1,373 @@
+// Dense (unquantized) matrices of the layer-list models: bfloat16 operands with fp32 accumulation on v_mfma_f32_16x16x32_bf16, or
+// fp32 throughout on v_mfma_f32_16x16x4_f32 (one rounding per product, fp32 adds: a true fp32 product, no reduced-precision mode).
+//   dense_mm_kernel<WT>   tiled mat-mul, 64 tokens x 64 outputs per work-group of four waves, any T / N / K (edges zero-filled)
+//   dense_mv_kernel<WT,C> a few tokens (C <= 8 columns): the activation rows live in LDS, a wave streams four weight rows at a time
+// Both take the same operand description (ps_seq.h psk_dense_args): ring rows, the token-shift mix and the epilogue
+// (bias, xIELU / tanh, scale) are part of the launch, so no mixer needs a kernel of its own around its projections.
+#include "ps_seq.h"
+
+#include <cmath>
+
+typedef float dn_f4 __attribute__((ext_vector_type(4)));
+typedef __bf16 dn_bf8 __attribute__((ext_vector_type(8)));
+typedef unsigned short dn_us8 __attribute__((ext_vector_type(8)));
+
+static __device__ __forceinline__ unsigned short dn_f2bf(float f) { // round to nearest even
+    unsigned u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (unsigned short)(u >> 16);
+}
+static __device__ __forceinline__ float dn_bf2f(unsigned short b) { return __uint_as_float((unsigned)b << 16); }
+
+struct dn_args {
+    const void *w;
+    const float *a;
+    long long lda, a_row0, a_mod;
+    const ps_seq_step *a_step;
+    int T;
+    long long N, K;
+    float *out;
+    long long ldo;
+    const float *bias;
+    int act;
+    float act_p, act_q, alpha;
+    const float *mu, *shift0;
+};
+
+// rows of A that exist and where they start (ring rows relative to the step's position)
+static __device__ __forceinline__ void dn_rows(const dn_args &g, long long &row0, int &T) {
+    row0 = g.a_row0;
+    T = g.T;
+    if (g.a_step) {
+        const long long p = g.a_step->pos0 + g.a_row0;
+        row0 = p > 0 ? p : 0;
+        const long long have = g.a_step->pos0 + g.a_step->n - row0;
+        if (have < T) T = (int)have;
+    }
+}
+static __device__ __forceinline__ const float *dn_arow(const dn_args &g, long long row0, int t) {
+    long long r = row0 + t;
+    if (g.a_mod > 0) r %= g.a_mod;
+    return g.a + r * g.lda;
+}
+static __device__ __forceinline__ float dn_aval(const dn_args &g, long long row0, int t, long long k) {
+    const float x = dn_arow(g, row0, t)[k];
+    if (!g.mu) return x;
+    const float p = t ? dn_arow(g, row0, t - 1)[k] : g.shift0[k];
+    return x + (p - x) * g.mu[k];
+}
+static __device__ __forceinline__ float dn_epi(const dn_args &g, float acc, long long n) {
+    if (g.bias) acc += g.bias[n];
+    if (g.act == PSD_ACT_XIELU) {
+        if (acc > 0.f) acc = g.act_p * acc * acc + 0.5f * acc;
+        else acc = g.act_q * (expm1f(acc) - acc) + 0.5f * acc;
+    } else if (g.act == PSD_ACT_TANH) {
+        acc = tanhf(acc);
+    }
+    return acc * g.alpha;
+}
+
+// ---------------------------------------------------------------------------------------------------- tiled mat-mul
+template <typename WT> struct dn_tile;
+template <> struct dn_tile<unsigned short> { static constexpr int BK = 32, LD = 40; typedef unsigned short S; }; // LDS rows padded to 80 B
+template <> struct dn_tile<float> { static constexpr int BK = 16, LD = 20; typedef float S; };
+
+template <typename WT>
+__global__ __launch_bounds__(256) void dense_mm_kernel(dn_args g) {
+    constexpr int BK = dn_tile<WT>::BK, LD = dn_tile<WT>::LD;
+    typedef typename dn_tile<WT>::S S;
+    __shared__ __attribute__((aligned(16))) S As[64 * LD];
+    __shared__ __attribute__((aligned(16))) S Bs[64 * LD];
+    long long row0;
+    int T;
+    dn_rows(g, row0, T);
+    const int t0 = blockIdx.y * 64;
+    if (t0 >= T) return; // (uniform per work-group: no barrier is skipped by part of it)
+    const long long n0 = (long long)blockIdx.x * 64;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+    const int lr = lane & 15, lq = lane >> 4;
+    const WT *W = (const WT *)g.w;
+    dn_f4 acc[2][2];
+    for (int i = 0; i < 2; i++)
+        for (int j = 0; j < 2; j++) acc[i][j] = dn_f4{0.f, 0.f, 0.f, 0.f};
+    constexpr int PER = 64 * BK / 256; // elements of each tile a thread stages: 8 (bf16) or 4 (fp32)
+    const int srow = tid / (BK / PER), sk = (tid % (BK / PER)) * PER;
+    for (long long k0 = 0; k0 < g.K; k0 += BK) {
+        { // A: tokens t0 .. t0+63
+            const int t = t0 + srow;
+            S tmp[PER];
+#pragma unroll
+            for (int e = 0; e < PER; e++) {
+                const long long k = k0 + sk + e;
+                const float v = (t < T && k < g.K) ? dn_aval(g, row0, t, k) : 0.f;
+                if constexpr (sizeof(WT) == 2) tmp[e] = dn_f2bf(v);
+                else tmp[e] = v;
+            }
+#pragma unroll
+            for (int e = 0; e < PER; e++) As[srow * LD + sk + e] = tmp[e];
+        }
+        { // B: weight rows n0 .. n0+63
+            const long long n = n0 + srow;
+            const long long k = k0 + sk;
+            S tmp[PER];
+            if (n < g.N && k + PER <= g.K && ((g.K * (long long)sizeof(WT)) % 16 == 0)) {
+                const dn_f4 raw = *(const dn_f4 *)(W + n * g.K + k); // 16 bytes: 8 bf16 or 4 floats
+                __builtin_memcpy(tmp, &raw, 16);
+            } else {
+#pragma unroll
+                for (int e = 0; e < PER; e++) tmp[e] = (n < g.N && k + e < g.K) ? W[n * g.K + k + e] : (S)0;
+            }
+#pragma unroll
+            for (int e = 0; e < PER; e++) Bs[srow * LD + sk + e] = tmp[e];
+        }
+        __syncthreads();
+        if constexpr (sizeof(WT) == 2) {
+            dn_bf8 fa[2], fb[2];
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                dn_us8 ra = *(const dn_us8 *)&As[(wm * 32 + i * 16 + lr) * LD + lq * 8];
+                dn_us8 rb = *(const dn_us8 *)&Bs[(wn * 32 + i * 16 + lr) * LD + lq * 8];
+                __builtin_memcpy(&fa[i], &ra, 16);
+                __builtin_memcpy(&fb[i], &rb, 16);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        } else {
+#pragma unroll
+            for (int kk = 0; kk < BK; kk += 4) {
+                float fa[2], fb[2];
+#pragma unroll
+                for (int i = 0; i < 2; i++) {
+                    fa[i] = As[(wm * 32 + i * 16 + lr) * LD + kk + lq];
+                    fb[i] = Bs[(wn * 32 + i * 16 + lr) * LD + kk + lq];
+                }
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int t = t0 + wm * 32 + i * 16 + lq * 4 + e;
+                const long long n = n0 + wn * 32 + j * 16 + lr;
+                if (t < T && n < g.N) g.out[(long long)t * g.ldo + n] = dn_epi(g, acc[i][j][e], n);
+            }
+}
+
+// ---------------------------------------------------------------------------------------------------- a few tokens: mat-vec
+// Dynamic LDS: C rows of K activations, as bf16-rounded fp32 values (bf16 mode: the same operand rounding as the tiled kernel) or fp32.
+template <typename WT, int C>
+__global__ __launch_bounds__(256) void dense_mv_kernel(dn_args g) {
+    extern __shared__ __attribute__((aligned(16))) float xs[]; // [C][Kp]
+    long long row0;
+    int T;
+    dn_rows(g, row0, T);
+    const long long K = g.K, Kp = (K + 7) / 8 * 8;
+    for (long long i = threadIdx.x; i < (long long)C * Kp; i += 256) {
+        const int c = (int)(i / Kp);
+        const long long k = i % Kp;
+        float v = (c < T && k < K) ? dn_aval(g, row0, c, k) : 0.f;
+        if constexpr (sizeof(WT) == 2) v = dn_bf2f(dn_f2bf(v));
+        xs[i] = v;
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const WT *W = (const WT *)g.w;
+    constexpr int RW = 4, VE = 16 / (int)sizeof(WT); // rows per wave at a time; elements per 16-byte load
+    const bool vec = (K * (long long)sizeof(WT)) % 16 == 0;
+    for (long long nb = ((long long)blockIdx.x * 4 + wave) * RW; nb < g.N; nb += (long long)gridDim.x * 4 * RW) {
+        float acc[RW][C];
+#pragma unroll
+        for (int r = 0; r < RW; r++)
+#pragma unroll
+            for (int c = 0; c < C; c++) acc[r][c] = 0.f;
+        if (vec) {
+            for (long long k = (long long)lane * VE; k < K; k += 64 * VE) {
+                dn_f4 raw[RW];
+#pragma unroll
+                for (int r = 0; r < RW; r++) {
+                    const long long n = nb + r < g.N ? nb + r : g.N - 1;
+                    raw[r] = __builtin_nontemporal_load((const dn_f4 *)(W + n * K + k));
+                }
+#pragma unroll
+                for (int r = 0; r < RW; r++) {
+                    float wv[VE];
+                    if constexpr (sizeof(WT) == 2) {
+                        unsigned short h[8];
+                        __builtin_memcpy(h, &raw[r], 16);
+#pragma unroll
+                        for (int e = 0; e < 8; e++) wv[e] = dn_bf2f(h[e]);
+                    } else {
+                        __builtin_memcpy(wv, &raw[r], 16);
+                    }
+#pragma unroll
+                    for (int c = 0; c < C; c++) {
+                        const float *x = xs + (long long)c * Kp + k;
+#pragma unroll
+                        for (int e = 0; e < VE; e++) acc[r][c] = fmaf(wv[e], x[e], acc[r][c]);
+                    }
+                }
+            }
+        } else {
+            for (long long k = lane; k < K; k += 64)
+#pragma unroll
+                for (int r = 0; r < RW; r++) {
+                    const long long n = nb + r < g.N ? nb + r : g.N - 1;
+                    float wv;
+                    if constexpr (sizeof(WT) == 2) wv = dn_bf2f(((const unsigned short *)W)[n * K + k]);
+                    else wv = ((const float *)W)[n * K + k];
+#pragma unroll
+                    for (int c = 0; c < C; c++) acc[r][c] = fmaf(wv, xs[(long long)c * Kp + k], acc[r][c]);
+                }
+        }
+#pragma unroll
+        for (int r = 0; r < RW; r++)
+#pragma unroll
+            for (int c = 0; c < C; c++) {
+                float v = acc[r][c];
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+                if (lane == 0 && nb + r < g.N && c < T) g.out[(long long)c * g.ldo + nb + r] = dn_epi(g, v, nb + r);
+            }
+    }
+}
+
+template <typename WT, int C>
+static void dn_launch_mv(hipStream_t st, const dn_args &g) {
+    const size_t lds = (size_t)C * ((g.K + 7) / 8 * 8) * 4;
+    static unsigned long long mask = 0;
+    if (ps_first_on_device(&mask)) (void)hipFuncSetAttribute((const void *)dense_mv_kernel<WT, C>, hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+    long long blocks = (g.N + 15) / 16;
+    if (blocks > 2048) blocks = 2048;
+    hipLaunchKernelGGL((dense_mv_kernel<WT, C>), dim3((unsigned)blocks), dim3(256), lds, st, g);
+}
+
+int psk_dense(hipStream_t st, const psk_dense_args &a) {
+    if (!a.w || a.T <= 0) return 0;
+    dn_args g;
+    g.w = a.w->data; g.a = a.a; g.lda = a.lda; g.a_row0 = a.a_row0; g.a_mod = a.a_mod; g.a_step = a.a_step; g.T = a.T;
+    g.N = a.w->N; g.K = a.w->K; g.out = a.out; g.ldo = a.ldo; g.bias = a.bias; g.act = a.act; g.act_p = a.act_p; g.act_q = a.act_q;
+    g.alpha = a.alpha; g.mu = a.mu; g.shift0 = a.shift0;
+    const bool bf = a.w->dtype == PS_BF16;
+    const size_t kp4 = (size_t)((g.K + 7) / 8 * 8) * 4;
+    if (!a.force_tiled && a.T <= 8) {
+        const int C = a.T <= 1 ? 1 : a.T <= 2 ? 2 : a.T <= 4 ? 4 : 8;
+        if (kp4 * C <= 64 * 1024) {
+            if (bf) {
+                if (C == 1) dn_launch_mv<unsigned short, 1>(st, g);
+                else if (C == 2) dn_launch_mv<unsigned short, 2>(st, g);
+                else if (C == 4) dn_launch_mv<unsigned short, 4>(st, g);
+                else dn_launch_mv<unsigned short, 8>(st, g);
+            } else {
+                if (C == 1) dn_launch_mv<float, 1>(st, g);
+                else if (C == 2) dn_launch_mv<float, 2>(st, g);
+                else if (C == 4) dn_launch_mv<float, 4>(st, g);
+                else dn_launch_mv<float, 8>(st, g);
+            }
+            return 0;
+        }
+    }
+    dim3 grid((unsigned)((g.N + 63) / 64), (unsigned)((a.T + 63) / 64));
+    if (bf) hipLaunchKernelGGL(dense_mm_kernel<unsigned short>, grid, dim3(256), 0, st, g);
+    else hipLaunchKernelGGL(dense_mm_kernel<float>, grid, dim3(256), 0, st, g);
+    return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------- upload, embedding, arg-max
+__global__ void dense_widen_kernel(const unsigned short *in, long long n, float *out) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) out[i] = dn_bf2f(in[i]);
+}
+void psk_dense_widen(hipStream_t st, const uint16_t *bf16, int64_t n, float *out) {
+    long long blocks = (n + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(dense_widen_kernel, dim3((unsigned)blocks), dim3(256), 0, st, bf16, (long long)n, out);
+}
+
+__global__ void dense_embed_kernel(const void *table, int is_bf16, long long K, const int32_t *tokens, const ps_seq_step *step, float *out, long long ldo) {
+    const int t = blockIdx.x;
+    const long long tok = (tokens ? tokens[t] : step->token0);
+    for (long long k = threadIdx.x; k < K; k += blockDim.x)
+        out[t * ldo + k] = is_bf16 ? dn_bf2f(((const unsigned short *)table)[tok * K + k]) : ((const float *)table)[tok * K + k];
+}
+void psk_embed(hipStream_t st, const ps_dense *table, const int32_t *tokens, const ps_seq_step *step, int T, float *out, int64_t ldo) {
+    hipLaunchKernelGGL(dense_embed_kernel, dim3(T), dim3(256), 0, st, table->data, table->dtype == PS_BF16 ? 1 : 0, (long long)table->K, tokens, step, out,
+                       (long long)ldo);
+}
+
+__global__ __launch_bounds__(256) void dense_argmax_kernel(const float *x, long long n, int32_t *out) {
+    __shared__ float bv[256];
+    __shared__ long long bi[256];
+    const float *row = x + (long long)blockIdx.x * n;
+    float best = -INFINITY;
+    long long at = n;
+    for (long long i = threadIdx.x; i < n; i += 256) {
+        const float v = row[i];
+        if (v > best || (v == best && i < at)) { best = v; at = i; }
+    }
+    bv[threadIdx.x] = best;
+    bi[threadIdx.x] = at;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if ((int)threadIdx.x < s) {
+            const float v = bv[threadIdx.x + s];
+            const long long i = bi[threadIdx.x + s];
+            if (v > bv[threadIdx.x] || (v == bv[threadIdx.x] && i < bi[threadIdx.x])) { bv[threadIdx.x] = v; bi[threadIdx.x] = i; }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[blockIdx.x] = (int32_t)(bi[0] < n ? bi[0] : 0);
+}
+void psk_argmax_rows(hipStream_t st, const float *x, int64_t n, int rows, int32_t *out) {
+    hipLaunchKernelGGL(dense_argmax_kernel, dim3(rows), dim3(256), 0, st, x, (long long)n, out);
+}
+
+extern "C" {
+int ps_hip_dense_upload(ps_hip_ctx *c, const uint16_t *host, int64_t N, int64_t K, int as_f32, ps_dense **out) {
+    *out = nullptr;
+    if (N <= 0 || K <= 0) PS_FAIL(c, "dense_upload: empty matrix");
+    PS_CHECK(c, hipSetDevice(c->device));
+    auto w = new ps_dense();
+    w->N = N; w->K = K; w->dtype = as_f32 ? PS_F32 : PS_BF16;
+    const size_t n = (size_t)N * K;
+    uint16_t *raw = nullptr;
+    if (ps_dev_malloc((void **)&raw, n * 2 + 64) != hipSuccess) { delete w; PS_FAIL(c, "dense_upload: out of device memory"); }
+    if (hipMemcpyAsync(raw, host, n * 2, hipMemcpyHostToDevice, c->stream) != hipSuccess) { (void)ps_dev_free(raw); delete w; PS_FAIL(c, "dense_upload: copy"); }
+    if (as_f32) {
+        float *f = nullptr;
+        if (ps_dev_malloc((void **)&f, n * 4 + 64) != hipSuccess) { (void)ps_dev_free(raw); delete w; PS_FAIL(c, "dense_upload: out of device memory"); }
+        psk_dense_widen(c->stream, raw, (int64_t)n, f);
+        w->data = f;
+    } else {
+        w->data = raw;
+    }
+    hipError_t e = hipStreamSynchronize(c->stream);
+    if (as_f32) (void)ps_dev_free(raw);
+    if (e != hipSuccess) { (void)ps_dev_free(w->data); delete w; PS_FAIL(c, std::string("dense_upload: ") + hipGetErrorString(e)); }
+    *out = w;
+    return 0;
+}
+void ps_hip_dense_free(ps_hip_ctx *c, ps_dense *w) {
+    if (!w) return;
+    if (c) (void)hipStreamSynchronize(c->stream);
+    (void)ps_dev_free(w->data);
+    delete w;
+}
+int ps_hip_dense_matmul(ps_hip_ctx *c, const ps_dense *w, const float *x, int T, float *out, float alpha) {
+    if (!w || T <= 0) PS_FAIL(c, "dense_matmul: bad argument");
+    psk_dense_args a;
+    a.w = w; a.a = x; a.lda = w->K; a.T = T; a.out = out; a.ldo = w->N; a.alpha = alpha;
+    psk_dense(c->stream, a);
+    PS_CHECK(c, hipGetLastError());
+    return 0;
+}
+}

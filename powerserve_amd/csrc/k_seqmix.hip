@@ -1,0 +1,304 @@
+// Mechanisms of the layer-list models that are not matrix products: RMS norms (with the residual add), causal convolutions over time
+// with a per-sequence tail, and the two recurrent scans (wkv, gated delta rule).  Everything here is fp32.
+//
+// The scans: a head's state S [d][dv] is split by COLUMN over threads -- every column j evolves on its own in both recurrences
+// (S_ij <- decay S_ij + k_i x_j needs only column j) -- and each column over R lanes of 16 rows each, so a step is 16 fused
+// multiply-adds per lane and one R-lane butterfly; the per-token vectors of a head (r, k, decays; unit q and k) are staged eight tokens
+// at a time through LDS, where their per-token scalars are reduced once for all columns.
+#include "ps_seq.h"
+
+#include <cmath>
+
+static __device__ __forceinline__ float sq_block_sum(float v, float *red) { // 256 threads
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return red[0] + red[1] + red[2] + red[3];
+}
+static __device__ __forceinline__ float sq_silu(float x) { return x / (1.f + expf(-x)); }
+static __device__ __forceinline__ float sq_softplus(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+
+__global__ __launch_bounds__(256) void sq_rmsnorm_kernel(const float *x, long long ldx, const int32_t *idx, const float *w, float offset, float eps, long long n,
+                                                         float *y, long long ldy) {
+    __shared__ float red[4];
+    const long long r = idx ? idx[blockIdx.x] : blockIdx.x;
+    const float *xr = x + r * ldx;
+    float s = 0.f;
+    for (long long i = threadIdx.x; i < n; i += 256) s += xr[i] * xr[i];
+    s = sq_block_sum(s, red);
+    const float inv = 1.f / sqrtf(s / (float)n + eps);
+    float *yr = y + (long long)blockIdx.x * ldy;
+    for (long long i = threadIdx.x; i < n; i += 256) yr[i] = xr[i] * inv * (offset + w[i]);
+}
+void psk_rmsnorm(hipStream_t st, const float *x, int64_t ldx, const int32_t *idx, const float *w, float offset, float eps, int64_t n, int rows, float *y, int64_t ldy) {
+    if (rows <= 0) return;
+    hipLaunchKernelGGL(sq_rmsnorm_kernel, dim3(rows), dim3(256), 0, st, x, (long long)ldx, idx, w, offset, eps, (long long)n, y, (long long)ldy);
+}
+
+__global__ __launch_bounds__(256) void sq_norm_residual_kernel(float *x, const float *y, const float *w, float offset, float eps, long long n) {
+    __shared__ float red[4];
+    const float *yr = y + (long long)blockIdx.x * n;
+    float *xr = x + (long long)blockIdx.x * n;
+    float s = 0.f;
+    for (long long i = threadIdx.x; i < n; i += 256) s += yr[i] * yr[i];
+    s = sq_block_sum(s, red);
+    const float inv = 1.f / sqrtf(s / (float)n + eps);
+    for (long long i = threadIdx.x; i < n; i += 256) xr[i] += yr[i] * inv * (offset + w[i]);
+}
+void psk_norm_residual(hipStream_t st, float *x, const float *y, const float *w, float offset, float eps, int64_t n, int rows) {
+    if (rows <= 0) return;
+    hipLaunchKernelGGL(sq_norm_residual_kernel, dim3(rows), dim3(256), 0, st, x, y, w, offset, eps, (long long)n);
+}
+
+// ---------------------------------------------------------------------------------------------------- causal convolution with a tail
+#define SQ_CONV_CHUNK 32
+static __device__ __forceinline__ void sq_conv_tail(float *tail, const float *in, long long ldi, int taps, long long C, int T, long long c) {
+    // new tail row i = input of token T - (taps-1) + i; before this step's first token: the old tail's row T + i (ascending i never reads a row already written)
+    for (int i = 0; i < taps - 1; i++) {
+        const int r = T + i - (taps - 1);
+        tail[(long long)i * C + c] = r >= 0 ? in[(long long)r * ldi + c] : tail[(long long)(T + i) * C + c];
+    }
+}
+__global__ __launch_bounds__(256) void sq_conv_kernel(const ps_seq_step *step, long long tail_off, const float *in, long long ldi, const float *w, int taps, int mode,
+                                                      long long C, int T, float *out, long long ldo) {
+    const long long c = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    float *tail = step->state + tail_off;
+    const int tb = blockIdx.y * SQ_CONV_CHUNK, te = min(T, tb + SQ_CONV_CHUNK);
+    for (int t = tb; t < te; t++) {
+        float s = 0.f;
+        for (int j = 0; j < taps; j++) {
+            const int r = t - taps + 1 + j;
+            const float v = r >= 0 ? in[(long long)r * ldi + c] : tail[(long long)(taps - 1 + r) * C + c];
+            s = fmaf(w[c * taps + j], v, s);
+        }
+        out[(long long)t * ldo + c] = mode == 0 ? in[(long long)t * ldi + c] + s : sq_silu(s);
+    }
+    if (gridDim.y == 1) sq_conv_tail(tail, in, ldi, taps, C, T, c); // one thread owns the channel: it has read what it overwrites
+}
+__global__ __launch_bounds__(256) void sq_conv_tail_kernel(const ps_seq_step *step, long long tail_off, const float *in, long long ldi, int taps, long long C, int T) {
+    const long long c = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (c < C) sq_conv_tail(step->state + tail_off, in, ldi, taps, C, T, c);
+}
+void psk_causal_conv(hipStream_t st, const ps_seq_step *step, int64_t tail_off, const float *in, int64_t ldi, const float *w, int taps, int mode, int64_t C, int T,
+                     float *out, int64_t ldo) {
+    const unsigned gx = (unsigned)((C + 255) / 256), gy = (unsigned)((T + SQ_CONV_CHUNK - 1) / SQ_CONV_CHUNK);
+    hipLaunchKernelGGL(sq_conv_kernel, dim3(gx, gy), dim3(256), 0, st, step, (long long)tail_off, in, (long long)ldi, w, taps, mode, (long long)C, T, out, (long long)ldo);
+    if (gy > 1 && taps > 1) hipLaunchKernelGGL(sq_conv_tail_kernel, dim3(gx), dim3(256), 0, st, step, (long long)tail_off, in, (long long)ldi, taps, (long long)C, T);
+}
+
+__global__ void sq_state_store_kernel(const ps_seq_step *step, long long off, const float *src, long long n) {
+    float *dst = step->state + off;
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) dst[i] = src[i];
+}
+void psk_state_store(hipStream_t st, const ps_seq_step *step, int64_t off, const float *src, int64_t n) {
+    hipLaunchKernelGGL(sq_state_store_kernel, dim3((unsigned)min((long long)((n + 255) / 256), 1024ll)), dim3(256), 0, st, step, (long long)off, src, (long long)n);
+}
+__global__ void sq_fill_kernel(float *p, float v, long long n) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) p[i] = v;
+}
+void psk_fill(hipStream_t st, float *p, float v, int64_t n) {
+    if (n <= 0) return;
+    hipLaunchKernelGGL(sq_fill_kernel, dim3((unsigned)min((long long)((n + 255) / 256), 4096ll)), dim3(256), 0, st, p, v, (long long)n);
+}
+__global__ void sq_copy_kernel(const float *s, float *d, long long n) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) d[i] = s[i];
+}
+void psk_copy(hipStream_t st, const float *src, float *dst, int64_t n) {
+    if (n <= 0) return;
+    hipLaunchKernelGGL(sq_copy_kernel, dim3((unsigned)min((long long)((n + 255) / 256), 4096ll)), dim3(256), 0, st, src, dst, (long long)n);
+}
+
+// ---------------------------------------------------------------------------------------------------- recurrent scans
+#define SQ_NR 16 // state rows per lane
+#define SQ_TC 8  // tokens staged per round
+static inline int sq_lanes_per_col(int d) { int R = 1; while (R * SQ_NR < d) R *= 2; return R; }
+
+// LDS: rs, ks, ws [TC][dp] (dp = NR * R, rows >= d zero), sc [TC] (sum_i r_i bonus_i k_i)
+__global__ __launch_bounds__(256) void sq_wkv_scan_kernel(const ps_seq_step *step, long long state_off, const float *r, const float *k, const float *v, const float *z,
+                                                          long long ld, const float *bonus, int d, int R, int T, float *o, long long ldo) {
+    extern __shared__ float lds[];
+    const int dp = SQ_NR * R, cpb = 256 / R;
+    float *rs = lds, *ks = rs + SQ_TC * dp, *ws = ks + SQ_TC * dp, *sc = ws + SQ_TC * dp;
+    const int h = blockIdx.y, tid = threadIdx.x, s = tid % R, j = blockIdx.x * cpb + tid / R;
+    const bool col = j < d;
+    float *S0 = step->state + state_off + (long long)h * d * d;
+    float S[SQ_NR];
+#pragma unroll
+    for (int m = 0; m < SQ_NR; m++) {
+        const int i = s + R * m;
+        S[m] = (col && i < d) ? S0[(long long)i * d + j] : 0.f;
+    }
+    const long long hb = (long long)h * d;
+    for (int t0 = 0; t0 < T; t0 += SQ_TC) {
+        const int nt = min(SQ_TC, T - t0);
+        __syncthreads();
+        for (int x = tid; x < SQ_TC * dp; x += 256) {
+            const int t = x / dp, i = x % dp;
+            float a = 0.f, b = 0.f, c = 0.f;
+            if (t < nt && i < d) {
+                const long long at = (long long)(t0 + t) * ld + hb + i;
+                a = r[at];
+                b = k[at];
+                c = expf(-expf(z[at]));
+            }
+            rs[x] = a;
+            ks[x] = b;
+            ws[x] = c;
+        }
+        float vj[SQ_TC];
+#pragma unroll
+        for (int t = 0; t < SQ_TC; t++) vj[t] = (col && t < nt) ? v[(long long)(t0 + t) * ld + hb + j] : 0.f;
+        __syncthreads();
+        for (int t = tid >> 6; t < SQ_TC; t += 4) { // one wave per token
+            float a = 0.f;
+            for (int i = tid & 63; i < d; i += 64) a += rs[t * dp + i] * bonus[hb + i] * ks[t * dp + i];
+#pragma unroll
+            for (int x = 32; x > 0; x >>= 1) a += __shfl_xor(a, x, 64);
+            if ((tid & 63) == 0) sc[t] = a;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int t = 0; t < SQ_TC; t++) {
+            if (t < nt) {
+                const float *rt = rs + t * dp, *kt = ks + t * dp, *wt = ws + t * dp;
+                float p = 0.f;
+#pragma unroll
+                for (int m = 0; m < SQ_NR; m++) {
+                    const int i = s + R * m;
+                    p = fmaf(rt[i], S[m], p);
+                    S[m] = fmaf(wt[i], S[m], kt[i] * vj[t]);
+                }
+                for (int x = 1; x < R; x <<= 1) p += __shfl_xor(p, x, 64);
+                if (col && s == 0) o[(long long)(t0 + t) * ldo + hb + j] = fmaf(vj[t], sc[t], p);
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < SQ_NR; m++) {
+        const int i = s + R * m;
+        if (col && i < d) S0[(long long)i * d + j] = S[m];
+    }
+}
+void psk_wkv_scan(hipStream_t st, const ps_seq_step *step, int64_t state_off, const float *r, const float *k, const float *v, const float *z, int64_t ld,
+                  const float *bonus, int H, int d, int T, float *o, int64_t ldo) {
+    const int R = sq_lanes_per_col(d), cpb = 256 / R;
+    const size_t lds = (size_t)(3 * SQ_TC * SQ_NR * R + SQ_TC) * 4;
+    hipLaunchKernelGGL(sq_wkv_scan_kernel, dim3((d + cpb - 1) / cpb, H), dim3(256), lds, st, step, (long long)state_off, r, k, v, z, (long long)ld, bonus, d, R, T, o,
+                       (long long)ldo);
+}
+
+// LDS: qs, ks [TC][dp]; per token: g, beta, kq
+__global__ __launch_bounds__(256) void sq_delta_scan_kernel(const ps_seq_step *step, long long state_off, const float *q, const float *k, const float *v,
+                                                            const float *braw, const float *araw, long long ld, long long ldb, const float *a_log, const float *dt_bias, int H,
+                                                            int KH, int d, int dv, int R, int T, float *o, long long ldo) {
+    extern __shared__ float lds[];
+    const int dp = SQ_NR * R, cpb = 256 / R;
+    float *qs = lds, *ks = qs + SQ_TC * dp, *gs = ks + SQ_TC * dp, *bs = gs + SQ_TC, *kq = bs + SQ_TC;
+    const int h = blockIdx.y, tid = threadIdx.x, s = tid % R, j = blockIdx.x * cpb + tid / R;
+    const bool col = j < dv;
+    float *S0 = step->state + state_off + (long long)h * d * dv;
+    float S[SQ_NR];
+#pragma unroll
+    for (int m = 0; m < SQ_NR; m++) {
+        const int i = s + R * m;
+        S[m] = (col && i < d) ? S0[(long long)i * dv + j] : 0.f;
+    }
+    const long long qb = (long long)(h / (H / KH)) * d, vb = (long long)h * dv;
+    const float qscale = 1.f / sqrtf((float)d), na = -expf(a_log[h]), db = dt_bias[h];
+    for (int t0 = 0; t0 < T; t0 += SQ_TC) {
+        const int nt = min(SQ_TC, T - t0);
+        __syncthreads();
+        for (int x = tid; x < SQ_TC * dp; x += 256) {
+            const int t = x / dp, i = x % dp;
+            const bool in = t < nt && i < d;
+            qs[x] = in ? q[(long long)(t0 + t) * ld + qb + i] : 0.f;
+            ks[x] = in ? k[(long long)(t0 + t) * ld + qb + i] : 0.f;
+        }
+        if (tid < SQ_TC) {
+            const bool in = tid < nt;
+            gs[tid] = in ? expf(na * sq_softplus(araw[(long long)(t0 + tid) * ldb + h] + db)) : 1.f;
+            bs[tid] = in ? 1.f / (1.f + expf(-braw[(long long)(t0 + tid) * ldb + h])) : 0.f;
+        }
+        float vj[SQ_TC];
+#pragma unroll
+        for (int t = 0; t < SQ_TC; t++) vj[t] = (col && t < nt) ? v[(long long)(t0 + t) * ld + vb + j] : 0.f;
+        __syncthreads();
+        for (int t = tid >> 6; t < SQ_TC; t += 4) { // one wave per token: unit vectors, then k . q
+            float a = 0.f, b = 0.f;
+            for (int i = tid & 63; i < d; i += 64) {
+                a += qs[t * dp + i] * qs[t * dp + i];
+                b += ks[t * dp + i] * ks[t * dp + i];
+            }
+#pragma unroll
+            for (int x = 32; x > 0; x >>= 1) {
+                a += __shfl_xor(a, x, 64);
+                b += __shfl_xor(b, x, 64);
+            }
+            const float iq = qscale / sqrtf(a + 1e-6f), ik = 1.f / sqrtf(b + 1e-6f);
+            float c = 0.f;
+            for (int i = tid & 63; i < d; i += 64) {
+                const float qn = qs[t * dp + i] * iq, kn = ks[t * dp + i] * ik;
+                qs[t * dp + i] = qn;
+                ks[t * dp + i] = kn;
+                c += qn * kn;
+            }
+#pragma unroll
+            for (int x = 32; x > 0; x >>= 1) c += __shfl_xor(c, x, 64);
+            if ((tid & 63) == 0) kq[t] = c;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int t = 0; t < SQ_TC; t++) {
+            if (t < nt) {
+                const float *qt = qs + t * dp, *kt = ks + t * dp;
+                const float g = gs[t];
+                float p1 = 0.f, p2 = 0.f;
+#pragma unroll
+                for (int m = 0; m < SQ_NR; m++) {
+                    const int i = s + R * m;
+                    S[m] *= g;
+                    p1 = fmaf(kt[i], S[m], p1);
+                    p2 = fmaf(qt[i], S[m], p2);
+                }
+                for (int x = 1; x < R; x <<= 1) {
+                    p1 += __shfl_xor(p1, x, 64);
+                    p2 += __shfl_xor(p2, x, 64);
+                }
+                const float u = bs[t] * (vj[t] - p1);
+#pragma unroll
+                for (int m = 0; m < SQ_NR; m++) S[m] = fmaf(kt[s + R * m], u, S[m]);
+                if (col && s == 0) o[(long long)(t0 + t) * ldo + vb + j] = fmaf(u, kq[t], p2); // S_new^T q = (g S)^T q + u (k . q)
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < SQ_NR; m++) {
+        const int i = s + R * m;
+        if (col && i < d) S0[(long long)i * dv + j] = S[m];
+    }
+}
+void psk_delta_scan(hipStream_t st, const ps_seq_step *step, int64_t state_off, const float *q, const float *k, const float *v, const float *braw,
+                    const float *araw, int64_t ld, int64_t ldb, const float *a_log, const float *dt_bias, int H, int KH, int d, int dv, int T, float *o, int64_t ldo) {
+    const int R = sq_lanes_per_col(d), cpb = 256 / R;
+    const size_t lds = (size_t)(2 * SQ_TC * SQ_NR * R + 3 * SQ_TC) * 4;
+    hipLaunchKernelGGL(sq_delta_scan_kernel, dim3((dv + cpb - 1) / cpb, H), dim3(256), lds, st, step, (long long)state_off, q, k, v, braw, araw, (long long)ld, (long long)ldb, a_log,
+                       dt_bias, H, KH, d, dv, R, T, o, (long long)ldo);
+}
+
+__global__ __launch_bounds__(64) void sq_headnorm_gate_kernel(float *o, long long ldo, const float *g, long long ldg, const float *w, int w_stride, float eps, int dv) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    float *oh = o + (long long)t * ldo + (long long)h * dv;
+    const float *gh = g + (long long)t * ldg + (long long)h * dv, *wh = w + (long long)h * w_stride;
+    float s = 0.f;
+    for (int j = lane; j < dv; j += 64) s += oh[j] * oh[j];
+#pragma unroll
+    for (int x = 32; x > 0; x >>= 1) s += __shfl_xor(s, x, 64);
+    const float inv = 1.f / sqrtf(s / (float)dv + eps);
+    for (int j = lane; j < dv; j += 64) oh[j] = oh[j] * inv * wh[j] * sq_silu(gh[j]);
+}
+void psk_headnorm_gate(hipStream_t st, float *o, int64_t ldo, const float *g, int64_t ldg, const float *w, int w_stride, float eps, int H, int dv, int T) {
+    hipLaunchKernelGGL(sq_headnorm_gate_kernel, dim3(T, H), dim3(64), 0, st, o, (long long)ldo, g, (long long)ldg, w, w_stride, eps, dv);
+}

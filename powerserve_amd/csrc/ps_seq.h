@@ -1,0 +1,85 @@
+// Internal launchers of the layer-list models (include/ps_hip.h, "layer-list models"): dense mat-mul / mat-vec (k_dense.hip),
+// norms, causal convolutions, token-shift, recurrent scans (k_seqmix.hip), latent attention (k_latent.hip).  All enqueue on `st`;
+// none waits.  Activations are fp32 row-major [tokens][features] with an explicit row stride.
+#pragma once
+#include "ps_internal.h"
+
+struct ps_dense {
+    int dtype = PS_BF16; // PS_BF16 or PS_F32
+    int64_t N = 0, K = 0;
+    void *data = nullptr;
+};
+
+// What every kernel of a step reads from DEVICE memory, so that one captured launch sequence replays for any position and slot:
+//   pos0 = position of the step's first token, n = tokens in the step, state = the slot's state block
+struct ps_seq_step {
+    int64_t pos0;
+    int32_t n, slot;
+    float *state;
+    int32_t token0; // single-token steps: the token to embed (greedy decoding feeds its own arg-max back here)
+    int32_t _pad;
+};
+
+enum { PSD_ACT_NONE = 0, PSD_ACT_XIELU = 1, PSD_ACT_TANH = 2 };
+
+// out[t][n] = alpha * act(sum_k A(t, k) W[n][k] + bias[n]),  t < T
+//   A(t, k) = a[row(t)][k], row(t) = t, or (a_row0 + t) mod a_mod when a_mod > 0 (rows of a ring), or, where a_step is given, rows of the
+//   ring starting at the device-side a_step->pos0 + a_row0 (clamped at 0) -- see k_latent.hip;
+//   with mu: the token-shift mix a[t][k] + (prev(t)[k] - a[t][k]) * mu[k], prev(t) = t ? a[t-1] : shift0.
+// In the bf16 mode A is rounded to bfloat16 (nearest even) before the product; accumulation is fp32 in both modes.
+struct psk_dense_args {
+    const ps_dense *w = nullptr;
+    const float *a = nullptr;
+    int64_t lda = 0, a_row0 = 0, a_mod = 0;
+    const ps_seq_step *a_step = nullptr; // ring rows relative to the step's position (a_row0 = offset, usually negative)
+    int T = 0;
+    float *out = nullptr;
+    int64_t ldo = 0;
+    const float *bias = nullptr;
+    int act = PSD_ACT_NONE;
+    float act_p = 0.f, act_q = 0.f, alpha = 1.f; // xIELU: act_p = softplus(p), act_q = 1/2 + softplus(q)
+    const float *mu = nullptr, *shift0 = nullptr;
+    int force_tiled = 0; // 1: the tiled mat-mul also for a few rows (A/B against the mat-vec)
+};
+int psk_dense(hipStream_t st, const psk_dense_args &a);
+void psk_dense_widen(hipStream_t st, const uint16_t *bf16, int64_t n, float *out);
+// out[t][:] = table[token(t)][:]; tokens device int32 (step != NULL and T == 1: the token is step->token0)
+void psk_embed(hipStream_t st, const ps_dense *table, const int32_t *tokens, const ps_seq_step *step, int T, float *out, int64_t ldo);
+// out[r] = index of the first maximum of x[r][0..n)
+void psk_argmax_rows(hipStream_t st, const float *x, int64_t n, int rows, int32_t *out);
+
+// ---- k_seqmix.hip
+// y[r] = x[row(r)] / sqrt(mean(x^2) + eps) * (offset + w),  row(r) = idx ? idx[r] : r
+void psk_rmsnorm(hipStream_t st, const float *x, int64_t ldx, const int32_t *idx, const float *w, float offset, float eps, int64_t n, int rows, float *y, int64_t ldy);
+// x[r] += y[r] / sqrt(mean(y^2) + eps) * (offset + w)
+void psk_norm_residual(hipStream_t st, float *x, const float *y, const float *w, float offset, float eps, int64_t n, int rows);
+// Causal convolution over time on each channel, taps taken from the step's rows and, before them, from the sequence's tail (the last taps - 1
+// inputs of earlier steps, [taps - 1][C] at step->state + tail_off): out[t][c] = f(sum_j w[c][j] in(t - taps + 1 + j)[c]); mode 0: f = in(t) + sum
+// (a residual around the convolution), mode 1: f = silu(sum).  The tail is brought up to date behind it.
+void psk_causal_conv(hipStream_t st, const ps_seq_step *step, int64_t tail_off, const float *in, int64_t ldi, const float *w, int taps, int mode,
+                     int64_t C, int T, float *out, int64_t ldo);
+// state row copy: (step->state + off)[0..n) = src[0..n)
+void psk_state_store(hipStream_t st, const ps_seq_step *step, int64_t off, const float *src, int64_t n);
+void psk_fill(hipStream_t st, float *p, float v, int64_t n);
+void psk_copy(hipStream_t st, const float *src, float *dst, int64_t n);
+
+// wkv scan.  r, k, v, z: [T][H*d] (row stride ld), z = the decay's pre-activation (w = exp(-exp(z))); bonus [H*d]; state [H][d][d] fp32 at
+// step->state + state_off.  o[t][h][j] = sum_i r_i (S_ij + bonus_i k_i v_j), then S_ij = w_i S_ij + k_i v_j.
+void psk_wkv_scan(hipStream_t st, const ps_seq_step *step, int64_t state_off, const float *r, const float *k, const float *v, const float *z, int64_t ld,
+                  const float *bonus, int H, int d, int T, float *o, int64_t ldo);
+// gated delta rule scan.  q, k: [T][KH*d] after convolution + silu (unit-normalised here, q also times d^-1/2), v [T][H*dv] (row stride ld), braw / araw [T][H] (row stride ldb);
+// per head: g = exp(-exp(a_log) softplus(araw + dt_bias)), beta = sigmoid(braw); S = g S; u = beta (v - S^T k); S += k u^T; o = S^T q.
+void psk_delta_scan(hipStream_t st, const ps_seq_step *step, int64_t state_off, const float *q, const float *k, const float *v, const float *braw,
+                    const float *araw, int64_t ld, int64_t ldb, const float *a_log, const float *dt_bias, int H, int KH, int d, int dv, int T, float *o, int64_t ldo);
+// o[t][h][:] = o / sqrt(mean_j o^2 + eps) * w(h, :) * silu(g[t][h][:]);  w_stride = dv (a weight per head) or 0 (one shared by the heads)
+void psk_headnorm_gate(hipStream_t st, float *o, int64_t ldo, const float *g, int64_t ldg, const float *w, int w_stride, float eps, int H, int dv, int T);
+
+// ---- k_latent.hip
+// One token per block.  y[t] = [ dq (q_rank) | ckv (kv_rank) | kr (rot_dim) ]:  cq[t] = rmsnorm(dq) * qnorm;  ring row (pos mod cap):
+// c = rmsnorm(ckv) * kvnorm, kr with its first rot_dims numbers rotated at pos (pairs (i, i + rot_dims/2), angle pos * freq[i]).  Ring at step->state + ring_off: [cap][kv_rank + rot_dim].
+void psk_latent_prep(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, const float *y, int64_t ldy, const float *qnorm, const float *kvnorm,
+                     float eps, int q_rank, int kv_rank, int rot_dim, int rot_dims, const float *freq, int T, float *cq, int64_t ldcq);
+// Windowed soft-max attention over expanded keys / values.  q [T][H*(d+dr)] (rotated part not yet rotated), kv [Nw][H*d + H*dv] for the positions
+// first .. first + Nw - 1 where first = max(0, pos0 - window + 1) (the caller expands exactly these ring rows), rotated key parts from the ring.
+void psk_latent_attn(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, const float *q, int64_t ldq, const float *kv, int64_t ldkv,
+                     const float *freq, int H, int d, int dr, int rot_dims, int dv, int kv_rank, int window, float scale, int T, float *o, int64_t ldo);

@@ -1,0 +1,384 @@
+// Layer-list models (include/ps_hip.h, "layer-list models"): the model object, its pool of sequence states and the step function.
+//
+// A step takes the next n tokens of ONE sequence from the state earlier steps left in its slot.  The residual stream is fp32; every
+// layer is  x += norm_b(mixer(conv(norm(x))))  then, where it has a feed-forward,  x += norm_b(ff(conv(norm(x)))).  What a sequence
+// carries: per layer the tails of the two input convolutions, and per mixer kind a token-shift row + the wkv state, the short
+// convolutions' tail + the delta-rule state, or the ring of latents -- one fp32 block per slot, rings last, the rest zeroed when
+// the slot is handed out.
+#include "ps_seq.h"
+
+#include <cmath>
+#include <cstring>
+#include <map>
+#include <string>
+#include <vector>
+
+namespace {
+struct LayerPlan {
+    ps_seq_layer d;
+    int64_t off_canon1 = 0, off_canon2 = 0, off_shift = 0, off_conv = 0, off_S = 0, off_ring = 0;
+    int cap = 0;          // latent: ring rows
+    float *freq = nullptr; // latent: rot_dim / 2 angular frequencies
+    float act_p = 0.f, act_q = 0.f;
+    int64_t ncat = 0, cqkv = 0;
+};
+} // namespace
+
+struct ps_hip_seq {
+    ps_hip_ctx *ctx = nullptr;
+    ps_seq_desc d;
+    std::vector<LayerPlan> L;
+    int64_t state_floats = 0, zero_floats = 0;
+    std::vector<float *> slot_state;
+    std::vector<int64_t> slot_pos; // -1: free
+    ps_seq_step *step = nullptr;   // device
+    float *x = nullptr, *hn = nullptr, *h = nullptr, *y = nullptr, *t1 = nullptr, *t2 = nullptr, *t3 = nullptr, *t4 = nullptr, *kvx = nullptr, *xn = nullptr,
+          *logits = nullptr;
+    int32_t *tokens = nullptr, *want = nullptr, *amax = nullptr, *ids = nullptr;
+    int ids_cap = 0;
+    int64_t n_t2q = 0; // t2: [max_batch][q_rank max] then the queries
+    float *dbg_layers = nullptr;
+    int mode = 0;
+    std::map<int, hipGraphExec_t> graphs; // single-token greedy step, per slot
+    uint64_t weight_bytes = 0;
+    std::vector<void *> owned;
+};
+
+__global__ void seq_set_step_kernel(ps_seq_step *s, long long pos0, int n, int slot, float *state, int token0) {
+    s->pos0 = pos0; s->n = n; s->slot = slot; s->state = state; s->token0 = token0; s->_pad = 0;
+}
+// behind a greedy single-token step: the arg-max becomes the next token, the position moves on, the id is kept at ids[_pad++]
+__global__ void seq_advance_kernel(ps_seq_step *s, const int32_t *amax, int32_t *ids) {
+    const int32_t id = amax[0];
+    ids[s->_pad] = id;
+    s->_pad += 1;
+    s->token0 = id;
+    s->pos0 += 1;
+}
+
+static int seq_fail(ps_hip_ctx *c, const std::string &msg) { c->err = msg; return 2; }
+
+static uint64_t dense_bytes(const ps_dense *w) { return w ? (uint64_t)w->N * w->K * (w->dtype == PS_BF16 ? 2 : 4) : 0; }
+
+extern "C" {
+
+int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) {
+    *out = nullptr;
+    if (!desc || desc->n_layers <= 0 || desc->width <= 0 || desc->vocab <= 0 || desc->max_batch <= 0 || desc->n_slots <= 0 || desc->canon_taps < 1)
+        return seq_fail(c, "seq_create: bad descriptor");
+    if (!desc->embed || !desc->head || !desc->final_norm) return seq_fail(c, "seq_create: embed / head / final_norm missing");
+    if (desc->embed->K != desc->width || desc->head->K != desc->width || desc->head->N != desc->vocab) return seq_fail(c, "seq_create: embed / head shape");
+    PS_CHECK(c, hipSetDevice(c->device));
+    auto m = new ps_hip_seq();
+    m->ctx = c;
+    m->d = *desc;
+    const int64_t W = desc->width, B = desc->max_batch;
+    int64_t off = 0, n1 = 0, n2 = 0, n3 = 0, n4 = 0, nkv = 0, nq = 0;
+    auto fail = [&](const std::string &msg) { ps_hip_seq_destroy(m); return seq_fail(c, "seq_create: " + msg); };
+    auto shape = [](const ps_dense *w, int64_t N, int64_t K) { return w && w->N == N && w->K == K; };
+    m->L.resize(desc->n_layers);
+    m->weight_bytes = dense_bytes(desc->head);
+    for (int i = 0; i < desc->n_layers; i++) {
+        LayerPlan &P = m->L[i];
+        P.d = desc->layers[i];
+        const ps_seq_layer &l = P.d;
+        const std::string at = "layer " + std::to_string(i) + ": ";
+        if (!l.norm1 || !l.norm1b || !l.canon1 || !l.out) return fail(at + "norm / canon / out missing");
+        P.off_canon1 = off; off += (int64_t)(desc->canon_taps - 1) * W;
+        if (l.ff_kind != PS_FF_NONE) {
+            if (l.ff_kind != PS_FF_DENSE_XIELU) return fail(at + "unknown feed-forward kind");
+            if (!l.norm2 || !l.norm2b || !l.canon2 || !shape(l.ff_up, l.ff, W) || !shape(l.ff_down, W, l.ff)) return fail(at + "feed-forward tensors");
+            P.off_canon2 = off; off += (int64_t)(desc->canon_taps - 1) * W;
+            const double sp = log1p(exp((double)l.ff_act_p)), sq = log1p(exp((double)l.ff_act_q));
+            P.act_p = (float)sp; P.act_q = (float)(0.5 + sq);
+            n4 = std::max<int64_t>(n4, l.ff);
+            m->weight_bytes += dense_bytes(l.ff_up) + dense_bytes(l.ff_down);
+        }
+        const int64_t H = l.heads, d = l.dim, dv = l.vdim;
+        if (H <= 0 || d <= 0) return fail(at + "heads / dim");
+        if (l.kind == PS_MIX_WKV) {
+            const int64_t Hd = H * d;
+            if (d > 256) return fail(at + "wkv: dim > 256 is not supported by the scan kernel");
+            if (!shape(l.in_r, Hd, W) || !shape(l.in_k, Hd, W) || !shape(l.in_v, Hd, W) || !shape(l.in_g, Hd, W) || !shape(l.decay1, l.decay_rank, W) ||
+                !shape(l.decay2, Hd, l.decay_rank) || !shape(l.out, W, Hd) || !l.mu || !l.decay0 || !l.bonus || !l.onorm)
+                return fail(at + "wkv tensors");
+            P.off_shift = off; off += W;
+            P.off_S = off; off += Hd * d;
+            n1 = std::max(n1, 5 * Hd);
+            n2 = std::max<int64_t>(n2, l.decay_rank);
+            n3 = std::max(n3, Hd);
+            m->weight_bytes += dense_bytes(l.in_r) * 4 + dense_bytes(l.decay1) + dense_bytes(l.decay2) + dense_bytes(l.out);
+        } else if (l.kind == PS_MIX_DELTA) {
+            if (d > 256) return fail(at + "delta: dim > 256 is not supported by the scan kernel");
+            if (l.kv_heads <= 0 || H % l.kv_heads || dv <= 0 || l.conv_taps < 1) return fail(at + "delta sizes");
+            P.cqkv = 2 * (int64_t)l.kv_heads * d + H * dv;
+            P.ncat = P.cqkv + H * dv + 2 * H;
+            if (!shape(l.in_cat, P.ncat, W) || !shape(l.out, W, H * dv) || !l.conv || !l.a_log || !l.dt_bias || !l.onorm) return fail(at + "delta tensors");
+            P.off_conv = off; off += (int64_t)(l.conv_taps - 1) * P.cqkv;
+            P.off_S = off; off += H * d * dv;
+            n1 = std::max(n1, P.ncat);
+            n2 = std::max(n2, P.cqkv);
+            n3 = std::max(n3, H * dv);
+            m->weight_bytes += dense_bytes(l.in_cat) + dense_bytes(l.out);
+        } else if (l.kind == PS_MIX_LATENT) {
+            if (dv <= 0 || dv > 256 || l.q_rank <= 0 || l.kv_rank <= 0 || l.rot_dim < 0 || l.rot_dims < 0 || l.rot_dims > l.rot_dim || (l.rot_dims & 1) || l.window < 1)
+                return fail(at + "latent sizes (vdim <= 256, even rot_dims <= rot_dim)");
+            P.ncat = (int64_t)l.q_rank + l.kv_rank + l.rot_dim;
+            if (!shape(l.in_cat, P.ncat, W) || !shape(l.uq, H * (d + l.rot_dim), l.q_rank) || !shape(l.ukv, H * d + H * dv, l.kv_rank) || !shape(l.out, W, H * dv) ||
+                !l.qnorm || !l.kvnorm)
+                return fail(at + "latent tensors");
+            P.cap = (int)(l.window - 1 + B);
+            n1 = std::max(n1, P.ncat);
+            nq = std::max(nq, H * (d + l.rot_dim));
+            m->n_t2q = std::max<int64_t>(m->n_t2q, l.q_rank);
+            n3 = std::max(n3, H * dv);
+            nkv = std::max(nkv, (int64_t)(l.window - 1 + B) * (H * d + H * dv));
+            m->weight_bytes += dense_bytes(l.in_cat) + dense_bytes(l.uq) + dense_bytes(l.ukv) + dense_bytes(l.out);
+        } else {
+            return fail(at + "unknown mixer kind");
+        }
+    }
+    n2 = std::max(n2, m->n_t2q + nq);
+    m->zero_floats = off;
+    for (auto &P : m->L)
+        if (P.d.kind == PS_MIX_LATENT) { P.off_ring = off; off += (int64_t)P.cap * (P.d.kv_rank + P.d.rot_dim); }
+    m->state_floats = off;
+    auto alloc = [&](void **p, size_t bytes) {
+        if (ps_dev_malloc(p, bytes + 256) != hipSuccess) return false;
+        m->owned.push_back(*p);
+        return true;
+    };
+    bool ok = true;
+    for (auto &P : m->L)
+        if (P.d.kind == PS_MIX_LATENT && P.d.rot_dims > 0) {
+            const int half = P.d.rot_dims / 2;
+            std::vector<float> f(half);
+            for (int i = 0; i < half; i++) f[i] = (float)pow((double)P.d.rot_base, -2.0 * i / (double)P.d.rot_dims);
+            ok = ok && alloc((void **)&P.freq, half * 4);
+            if (ok) ok = hipMemcpyAsync(P.freq, f.data(), half * 4, hipMemcpyHostToDevice, c->stream) == hipSuccess && hipStreamSynchronize(c->stream) == hipSuccess;
+        }
+    ok = ok && alloc((void **)&m->step, sizeof(ps_seq_step)) && alloc((void **)&m->x, B * W * 4) && alloc((void **)&m->hn, B * W * 4) && alloc((void **)&m->h, B * W * 4) &&
+         alloc((void **)&m->y, B * W * 4) && alloc((void **)&m->t1, B * std::max<int64_t>(n1, 1) * 4) && alloc((void **)&m->t2, B * std::max<int64_t>(n2, 1) * 4) &&
+         alloc((void **)&m->t3, B * std::max<int64_t>(n3, 1) * 4) && alloc((void **)&m->t4, B * std::max<int64_t>(n4, 1) * 4) &&
+         alloc((void **)&m->kvx, std::max<int64_t>(nkv, 1) * 4) && alloc((void **)&m->xn, B * W * 4) && alloc((void **)&m->logits, B * (int64_t)desc->vocab * 4) &&
+         alloc((void **)&m->tokens, B * 4) && alloc((void **)&m->want, B * 4) && alloc((void **)&m->amax, B * 4);
+    m->slot_state.assign(desc->n_slots, nullptr);
+    m->slot_pos.assign(desc->n_slots, -1);
+    for (int s = 0; ok && s < desc->n_slots; s++) ok = alloc((void **)&m->slot_state[s], (size_t)m->state_floats * 4);
+    if (!ok) return fail("out of device memory");
+    *out = m;
+    return 0;
+}
+
+void ps_hip_seq_destroy(ps_hip_seq *m) {
+    if (!m) return;
+    (void)hipSetDevice(m->ctx->device);
+    (void)hipStreamSynchronize(m->ctx->stream);
+    for (auto &g : m->graphs) (void)hipGraphExecDestroy(g.second);
+    for (void *p : m->owned) (void)ps_dev_free(p);
+    if (m->ids) (void)ps_dev_free(m->ids);
+    delete m;
+}
+
+int ps_hip_seq_acquire(ps_hip_seq *m, int *slot) {
+    ps_hip_ctx *c = m->ctx;
+    *slot = -1;
+    for (size_t s = 0; s < m->slot_pos.size(); s++)
+        if (m->slot_pos[s] < 0) {
+            psk_fill(c->stream, m->slot_state[s], 0.f, m->zero_floats); // (a fill kernel, not a memset: the state is read by captured launch sequences)
+            PS_CHECK(c, hipGetLastError());
+            m->slot_pos[s] = 0;
+            *slot = (int)s;
+            return 0;
+        }
+    return seq_fail(c, "seq_acquire: every slot is in use");
+}
+int ps_hip_seq_release(ps_hip_seq *m, int slot) {
+    if (slot < 0 || slot >= (int)m->slot_pos.size() || m->slot_pos[slot] < 0) return seq_fail(m->ctx, "seq_release: not a live slot");
+    m->slot_pos[slot] = -1;
+    return 0;
+}
+int64_t ps_hip_seq_position(const ps_hip_seq *m, int slot) { return (slot < 0 || slot >= (int)m->slot_pos.size()) ? -1 : m->slot_pos[slot]; }
+size_t ps_hip_seq_slot_bytes(const ps_hip_seq *m) { return (size_t)m->state_floats * 4; }
+uint64_t ps_hip_seq_weight_bytes_per_token(const ps_hip_seq *m) { return m->weight_bytes; }
+int ps_hip_seq_debug_layers(ps_hip_seq *m, float *buf) { m->dbg_layers = buf; return 0; }
+int ps_hip_seq_set_mode(ps_hip_seq *m, int mode) { m->mode = mode; return 0; }
+
+} // extern "C"
+
+// The launches of one portion: T <= max_batch tokens (device ids in m->tokens, or the step's own token0 when from_step) of the slot whose state
+// pointer is `state`.  kv_rows_hint < 0: the step's position is known on the host (pos0); >= 0: a captured sequence that must hold for any
+// position -- the window's expansion is launched for its most rows and cut on the device.
+static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool any_pos, bool from_step) {
+    hipStream_t st = m->ctx->stream;
+    const ps_seq_desc &D = m->d;
+    const int64_t W = D.width;
+    const bool tiled = (m->mode & 2) != 0;
+    psk_embed(st, D.embed, from_step ? nullptr : m->tokens, m->step, T, m->x, W);
+    auto mm = [&](const ps_dense *w, const float *a, int64_t lda, float *out, int64_t ldo) {
+        psk_dense_args g;
+        g.w = w; g.a = a; g.lda = lda; g.T = T; g.out = out; g.ldo = ldo; g.force_tiled = tiled;
+        return g;
+    };
+    for (int li = 0; li < D.n_layers; li++) {
+        const LayerPlan &P = m->L[li];
+        const ps_seq_layer &l = P.d;
+        const int64_t H = l.heads, d = l.dim, dv = l.vdim;
+        psk_rmsnorm(st, m->x, W, nullptr, l.norm1, D.norm_offset, D.norm_eps, W, T, m->hn, W);
+        psk_causal_conv(st, m->step, P.off_canon1, m->hn, W, l.canon1, D.canon_taps, 0, W, T, m->h, W);
+        if (l.kind == PS_MIX_WKV) {
+            const int64_t Hd = H * d, NW = 5 * Hd;
+            const ps_dense *ws[4] = {l.in_r, l.in_k, l.in_v, l.in_g};
+            for (int s = 0; s < 4; s++) {
+                auto g = mm(ws[s], m->h, W, m->t1 + s * Hd, NW);
+                g.mu = l.mu + s * W; g.shift0 = state + P.off_shift;
+                psk_dense(st, g);
+            }
+            {
+                auto g = mm(l.decay1, m->h, W, m->t2, l.decay_rank);
+                g.mu = l.mu + 4 * W; g.shift0 = state + P.off_shift; g.act = PSD_ACT_TANH;
+                psk_dense(st, g);
+                auto g2 = mm(l.decay2, m->t2, l.decay_rank, m->t1 + 4 * Hd, NW);
+                g2.bias = l.decay0;
+                psk_dense(st, g2);
+            }
+            psk_state_store(st, m->step, P.off_shift, m->h + (int64_t)(T - 1) * W, W);
+            psk_wkv_scan(st, m->step, P.off_S, m->t1, m->t1 + Hd, m->t1 + 2 * Hd, m->t1 + 4 * Hd, NW, l.bonus, (int)H, (int)d, T, m->t3, Hd);
+            psk_headnorm_gate(st, m->t3, Hd, m->t1 + 3 * Hd, NW, l.onorm, (int)d, D.norm_eps, (int)H, (int)d, T);
+            psk_dense(st, mm(l.out, m->t3, Hd, m->y, W));
+        } else if (l.kind == PS_MIX_DELTA) {
+            const int64_t KHd = (int64_t)l.kv_heads * d, Hv = H * dv;
+            psk_dense(st, mm(l.in_cat, m->h, W, m->t1, P.ncat));
+            psk_causal_conv(st, m->step, P.off_conv, m->t1, P.ncat, l.conv, l.conv_taps, 1, P.cqkv, T, m->t2, P.cqkv);
+            psk_delta_scan(st, m->step, P.off_S, m->t2, m->t2 + KHd, m->t2 + 2 * KHd, m->t1 + P.cqkv + Hv, m->t1 + P.cqkv + Hv + H, P.cqkv, P.ncat, l.a_log, l.dt_bias,
+                           (int)H, l.kv_heads, (int)d, (int)dv, T, m->t3, Hv);
+            psk_headnorm_gate(st, m->t3, Hv, m->t1 + P.cqkv, P.ncat, l.onorm, 0, D.norm_eps, (int)H, (int)dv, T);
+            psk_dense(st, mm(l.out, m->t3, Hv, m->y, W));
+        } else {
+            const int64_t dr = l.rot_dim, rs = l.kv_rank + dr, Hv = H * dv, nq = H * (d + dr);
+            float *cq = m->t2, *q = m->t2 + (int64_t)D.max_batch * m->n_t2q;
+            psk_dense(st, mm(l.in_cat, m->h, W, m->t1, P.ncat));
+            psk_latent_prep(st, m->step, P.off_ring, P.cap, m->t1, P.ncat, l.qnorm, l.kvnorm, D.norm_eps, l.q_rank, l.kv_rank, (int)dr, l.rot_dims, P.freq, T, cq, l.q_rank);
+            psk_dense(st, mm(l.uq, cq, l.q_rank, q, nq));
+            { // the window's keys and values, expanded from the ring rows  max(0, pos0 - window + 1) .. pos0 + T - 1
+                auto g = mm(l.ukv, state + P.off_ring, rs, m->kvx, H * d + Hv);
+                g.a_step = m->step; g.a_row0 = -(int64_t)(l.window - 1); g.a_mod = P.cap;
+                g.T = any_pos ? l.window - 1 + T : (int)(std::min<int64_t>(pos0, l.window - 1) + T);
+                g.force_tiled = 1;
+                psk_dense(st, g);
+            }
+            psk_latent_attn(st, m->step, P.off_ring, P.cap, q, nq, m->kvx, H * d + Hv, P.freq, (int)H, (int)d, (int)dr, l.rot_dims, (int)dv, l.kv_rank, l.window, l.scale, T, m->t3, Hv);
+            psk_dense(st, mm(l.out, m->t3, Hv, m->y, W));
+        }
+        psk_norm_residual(st, m->x, m->y, l.norm1b, D.norm_offset, D.norm_eps, W, T);
+        if (l.ff_kind == PS_FF_DENSE_XIELU) {
+            psk_rmsnorm(st, m->x, W, nullptr, l.norm2, D.norm_offset, D.norm_eps, W, T, m->hn, W);
+            psk_causal_conv(st, m->step, P.off_canon2, m->hn, W, l.canon2, D.canon_taps, 0, W, T, m->h, W);
+            auto g = mm(l.ff_up, m->h, W, m->t4, l.ff);
+            g.act = PSD_ACT_XIELU; g.act_p = P.act_p; g.act_q = P.act_q;
+            psk_dense(st, g);
+            psk_dense(st, mm(l.ff_down, m->t4, l.ff, m->y, W));
+            psk_norm_residual(st, m->x, m->y, l.norm2b, D.norm_offset, D.norm_eps, W, T);
+        }
+        if (m->dbg_layers && !any_pos) psk_copy(st, m->x, m->dbg_layers + (int64_t)li * D.max_batch * W, (int64_t)T * W);
+    }
+}
+
+// final norm on `rows` rows of x (idx: device indices, or NULL for rows 0 ..), logits, arg-max
+static void seq_head(ps_hip_seq *m, const int32_t *idx, int rows) {
+    hipStream_t st = m->ctx->stream;
+    const ps_seq_desc &D = m->d;
+    psk_rmsnorm(st, m->x, D.width, idx, D.final_norm, D.norm_offset, D.norm_eps, D.width, rows, m->xn, D.width);
+    psk_dense_args g;
+    g.w = D.head; g.a = m->xn; g.lda = D.width; g.T = rows; g.out = m->logits; g.ldo = D.vocab; g.alpha = D.logit_scale; g.force_tiled = (m->mode & 2) != 0;
+    psk_dense(st, g);
+    psk_argmax_rows(st, m->logits, D.vocab, rows, m->amax);
+}
+
+extern "C" {
+
+int ps_hip_seq_forward(ps_hip_seq *m, int slot, const int32_t *tokens, int n, const int32_t *want, int n_want, float *logits_host, int32_t *argmax_host) {
+    ps_hip_ctx *c = m->ctx;
+    if (slot < 0 || slot >= (int)m->slot_pos.size() || m->slot_pos[slot] < 0) return seq_fail(c, "seq_forward: not a live slot");
+    if (n <= 0 || !tokens) return seq_fail(c, "seq_forward: no tokens");
+    for (int i = 0; i < n; i++)
+        if (tokens[i] < 0 || tokens[i] >= m->d.vocab) return seq_fail(c, "seq_forward: token id outside the vocabulary");
+    for (int i = 0; i < n_want; i++)
+        if (want[i] < 0 || want[i] >= n || (i && want[i] < want[i - 1])) return seq_fail(c, "seq_forward: want must be ascending indices into the step's tokens");
+    PS_CHECK(c, hipSetDevice(c->device));
+    const int B = m->d.max_batch;
+    int wi = 0;
+    for (int t0 = 0; t0 < n; t0 += B) {
+        const int T = std::min(B, n - t0);
+        const int64_t pos0 = m->slot_pos[slot];
+        PS_CHECK(c, hipMemcpyAsync(m->tokens, tokens + t0, (size_t)T * 4, hipMemcpyHostToDevice, c->stream));
+        hipLaunchKernelGGL(seq_set_step_kernel, dim3(1), dim3(1), 0, c->stream, m->step, (long long)pos0, T, slot, m->slot_state[slot], (int)tokens[t0]);
+        seq_layers(m, m->slot_state[slot], T, pos0, false, false);
+        std::vector<int32_t> idx;
+        const int w0 = wi;
+        while (wi < n_want && want[wi] < t0 + T) idx.push_back(want[wi++] - t0);
+        if (!idx.empty()) {
+            PS_CHECK(c, hipMemcpyAsync(m->want, idx.data(), idx.size() * 4, hipMemcpyHostToDevice, c->stream));
+            seq_head(m, m->want, (int)idx.size());
+            if (logits_host)
+                PS_CHECK(c, hipMemcpyAsync(logits_host + (size_t)w0 * m->d.vocab, m->logits, idx.size() * (size_t)m->d.vocab * 4, hipMemcpyDeviceToHost, c->stream));
+            if (argmax_host) PS_CHECK(c, hipMemcpyAsync(argmax_host + w0, m->amax, idx.size() * 4, hipMemcpyDeviceToHost, c->stream));
+        }
+        PS_CHECK(c, hipStreamSynchronize(c->stream)); // (idx and the caller's token buffer are read by the copies above)
+        PS_CHECK(c, hipGetLastError());
+        m->slot_pos[slot] = pos0 + T;
+    }
+    return 0;
+}
+
+int ps_hip_seq_decode_greedy(ps_hip_seq *m, int slot, int32_t token, int steps, int32_t *out_ids) {
+    ps_hip_ctx *c = m->ctx;
+    if (slot < 0 || slot >= (int)m->slot_pos.size() || m->slot_pos[slot] < 0) return seq_fail(c, "seq_decode_greedy: not a live slot");
+    if (steps <= 0) return 0;
+    if (token < 0 || token >= m->d.vocab) return seq_fail(c, "seq_decode_greedy: token id outside the vocabulary");
+    PS_CHECK(c, hipSetDevice(c->device));
+    if (steps > m->ids_cap) {
+        if (m->ids) { PS_CHECK(c, hipStreamSynchronize(c->stream)); (void)ps_dev_free(m->ids); m->ids = nullptr; }
+        PS_CHECK(c, ps_dev_malloc((void **)&m->ids, (size_t)steps * 4 + 256));
+        m->ids_cap = steps;
+        for (auto &g : m->graphs) (void)hipGraphExecDestroy(g.second); // (the captured sequences hold the old pointer)
+        m->graphs.clear();
+    }
+    float *state = m->slot_state[slot];
+    hipLaunchKernelGGL(seq_set_step_kernel, dim3(1), dim3(1), 0, c->stream, m->step, (long long)m->slot_pos[slot], 1, slot, state, (int)token);
+    auto one = [&]() {
+        seq_layers(m, state, 1, 0, true, true);
+        seq_head(m, nullptr, 1);
+        hipLaunchKernelGGL(seq_advance_kernel, dim3(1), dim3(1), 0, c->stream, m->step, m->amax, m->ids);
+    };
+    if (m->mode & 1) {
+        for (int i = 0; i < steps; i++) one();
+    } else {
+        auto it = m->graphs.find(slot);
+        if (it == m->graphs.end()) {
+            hipGraph_t g = nullptr;
+            PS_CHECK(c, hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal));
+            one();
+            const hipError_t e = hipStreamEndCapture(c->stream, &g);
+            if (e != hipSuccess) { if (g) (void)hipGraphDestroy(g); return seq_fail(c, std::string("seq_decode_greedy: graph capture failed: ") + hipGetErrorString(e)); }
+            hipGraphExec_t ge = nullptr;
+            const hipError_t e2 = hipGraphInstantiate(&ge, g, nullptr, nullptr, 0);
+            (void)hipGraphDestroy(g);
+            if (e2 != hipSuccess) return seq_fail(c, std::string("seq_decode_greedy: graph instantiate failed: ") + hipGetErrorString(e2));
+            it = m->graphs.emplace(slot, ge).first;
+        }
+        for (int i = 0; i < steps; i++) PS_CHECK(c, hipGraphLaunch(it->second, c->stream));
+    }
+    PS_CHECK(c, hipMemcpyAsync(out_ids, m->ids, (size_t)steps * 4, hipMemcpyDeviceToHost, c->stream));
+    PS_CHECK(c, hipStreamSynchronize(c->stream));
+    PS_CHECK(c, hipGetLastError());
+    m->slot_pos[slot] += steps;
+    return 0;
+}
+
+int ps_hip_seq_bench_kernel(ps_hip_seq *m, int which, int T, int reps, double *us, double *bytes, double *flops) {
+    (void)m; (void)which; (void)T; (void)reps; (void)us; (void)bytes; (void)flops;
+    return seq_fail(m->ctx, "seq_bench_kernel: not built yet");
+}
+
+} // extern "C"

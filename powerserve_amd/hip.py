@@ -16,6 +16,7 @@ from . import gguf
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("PS_HIP_LIB") or os.path.join(HERE, "lib", "libps_hip.so")  # PS_HIP_LIB: an A/B build (tools/ab_build.py)
+SEQ_LIB_PATH = os.path.join(HERE, "lib", "libps_hip_seq.so")  # the context + the layer-list models only (powerserve_amd/build.py build_seq)
 
 F32, F16, Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, Q8_K, I32 = 0, 1, 2, 8, 12, 13, 14, 15, 26
 ATTN_TIMEOUT = 3  # PS_HIP_ATTN_TIMEOUT (include/ps_hip.h)
@@ -33,7 +34,15 @@ EXPORTS = [
     "ps_hip_model_forward", "ps_hip_model_decode_greedy", "ps_hip_model_logits", "ps_hip_model_scratch", "ps_hip_model_k_cache",
     "ps_hip_model_v_cache", "ps_hip_model_weight_bytes_per_token", "ps_hip_model_set_mode", "ps_hip_model_bench_gemv", "ps_hip_model_bench_matmul", "ps_hip_debug_timeline", "ps_hip_last_matmul_kernel", "ps_hip_debug_set", "ps_hip_debug_f16_gemm", "ps_hip_model_forward_tree", "ps_hip_model_prefill", "ps_hip_model_forward_lowered", "ps_hip_model_sync_check", "ps_hip_model_kv_mask",
     "ps_hip_soft_max", "ps_hip_model_kv_copy", "ps_hip_model_kv_save_tokens", "ps_hip_model_kv_unmask_tokens", "ps_hip_model_kv_append_tokens", "ps_hip_model_argmax",
+    "ps_hip_dense_upload", "ps_hip_dense_free", "ps_hip_dense_matmul", "ps_hip_seq_create", "ps_hip_seq_destroy", "ps_hip_seq_acquire", "ps_hip_seq_release",
+    "ps_hip_seq_position", "ps_hip_seq_slot_bytes", "ps_hip_seq_forward", "ps_hip_seq_decode_greedy", "ps_hip_seq_debug_layers", "ps_hip_seq_set_mode",
+    "ps_hip_seq_weight_bytes_per_token", "ps_hip_seq_bench_kernel",
 ]
+# the part of EXPORTS that lib/libps_hip_seq.so has (everything else belongs to the quantized path)
+SEQ_EXPORTS = [n for n in EXPORTS if n.startswith(("ps_hip_dense_", "ps_hip_seq_"))] + [
+    "ps_hip_abi_version", "ps_hip_device_count", "ps_hip_create", "ps_hip_destroy", "ps_hip_last_error", "ps_hip_device_name", "ps_hip_malloc", "ps_hip_free",
+    "ps_hip_memcpy_h2d", "ps_hip_memcpy_d2h", "ps_hip_memset", "ps_hip_sync", "ps_hip_stream", "ps_hip_event_create", "ps_hip_event_record",
+    "ps_hip_event_elapsed_ms", "ps_hip_event_destroy"]
 
 
 class PSTensor(C.Structure):
@@ -76,18 +85,38 @@ def make_config(d: dict) -> LLMConfig:
                      int(d["head_size"]), float(d["norm_eps"]), rp)
 
 
+class SeqLayer(C.Structure):
+    """ps_seq_layer (include/ps_hip.h)"""
+    _fields_ = ([(n, C.c_int32) for n in ("kind", "heads", "kv_heads", "dim", "vdim", "conv_taps", "decay_rank", "q_rank", "kv_rank", "rot_dim", "rot_dims", "window")] +
+                [("rot_base", C.c_float), ("scale", C.c_float), ("ff_kind", C.c_int32), ("ff", C.c_int32), ("ff_act_p", C.c_float), ("ff_act_q", C.c_float)] +
+                [(n, C.c_void_p) for n in ("norm1", "norm2", "norm1b", "norm2b", "canon1", "canon2")] +
+                [(n, C.c_void_p) for n in ("in_r", "in_k", "in_v", "in_g", "decay1", "decay2", "in_cat", "uq", "ukv", "out", "ff_up", "ff_down")] +
+                [(n, C.c_void_p) for n in ("mu", "decay0", "bonus", "onorm", "conv", "a_log", "dt_bias", "qnorm", "kvnorm")])
+
+
+class SeqDesc(C.Structure):
+    """ps_seq_desc (include/ps_hip.h)"""
+    _fields_ = ([(n, C.c_int32) for n in ("n_layers", "width", "vocab", "canon_taps", "max_batch", "n_slots", "compute")] +
+                [("norm_eps", C.c_float), ("norm_offset", C.c_float), ("logit_scale", C.c_float)] +
+                [("embed", C.c_void_p), ("head", C.c_void_p), ("final_norm", C.c_void_p), ("layers", C.POINTER(SeqLayer))])
+
+
 _LIB = None
 
 
-def lib() -> C.CDLL:
-    """Load libps_hip.so (raises if it has not been built: python -m powerserve_amd.build)."""
+def lib(seq_only_ok: bool = False) -> C.CDLL:
+    """Load libps_hip.so (raises if it has not been built: python -m powerserve_amd.build).  seq_only_ok: where the full library is not
+    there, lib/libps_hip_seq.so (the context and the layer-list models) will do."""
     global _LIB
     if _LIB is not None:
         return _LIB
-    if not os.path.exists(LIB_PATH):
-        raise RuntimeError(f"{LIB_PATH} is missing: the HIP backend is not built (run __graft_entry__.build()); "
+    path = LIB_PATH
+    if not os.path.exists(path) and seq_only_ok and os.path.exists(SEQ_LIB_PATH):
+        path = SEQ_LIB_PATH
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: the HIP backend is not built (run __graft_entry__.build()); "
                            "there is no CPU fallback")
-    L = C.CDLL(LIB_PATH)
+    L = C.CDLL(path)
     vp, i32, i64, sz = C.c_void_p, C.c_int, C.c_int64, C.c_size_t
     T = C.POINTER(PSTensor)
     sig = {
@@ -124,8 +153,18 @@ def lib() -> C.CDLL:
         "ps_hip_last_matmul_kernel": (C.c_char_p, []),
         "ps_hip_debug_set": (i32, [i32, i32]),
         "ps_hip_debug_f16_gemm": (i32, [vp, i32, C.c_int64, C.c_int64, i32, C.c_float, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+        "ps_hip_dense_upload": (i32, [vp, vp, i64, i64, i32, C.POINTER(vp)]), "ps_hip_dense_free": (None, [vp, vp]),
+        "ps_hip_dense_matmul": (i32, [vp, vp, vp, i32, vp, C.c_float]),
+        "ps_hip_seq_create": (i32, [vp, C.POINTER(SeqDesc), C.POINTER(vp)]), "ps_hip_seq_destroy": (None, [vp]),
+        "ps_hip_seq_acquire": (i32, [vp, C.POINTER(i32)]), "ps_hip_seq_release": (i32, [vp, i32]), "ps_hip_seq_position": (i64, [vp, i32]),
+        "ps_hip_seq_slot_bytes": (sz, [vp]), "ps_hip_seq_forward": (i32, [vp, i32, vp, i32, vp, i32, vp, vp]),
+        "ps_hip_seq_decode_greedy": (i32, [vp, i32, i32, i32, vp]), "ps_hip_seq_debug_layers": (i32, [vp, vp]), "ps_hip_seq_set_mode": (i32, [vp, i32]),
+        "ps_hip_seq_weight_bytes_per_token": (C.c_uint64, [vp]),
+        "ps_hip_seq_bench_kernel": (i32, [vp, i32, i32, i32, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     }
     for name, (res, args) in sig.items():
+        if path != LIB_PATH and name not in SEQ_EXPORTS:
+            continue
         fn = getattr(L, name)
         fn.restype, fn.argtypes = res, args
     _LIB = L
@@ -141,8 +180,8 @@ def _ptr(a: np.ndarray):
 
 
 class Ctx:
-    def __init__(self, device: int = 0):
-        self.L = lib()
+    def __init__(self, device: int = 0, seq_only_ok: bool = False):
+        self.L = lib(seq_only_ok)
         if self.L.ps_hip_device_count() <= 0:
             raise PSHipError("no HIP device visible: the MI355X backend cannot run (there is no CPU fallback)")
         h = C.c_void_p()

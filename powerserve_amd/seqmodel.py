@@ -1,0 +1,259 @@
+"""Layer-list models on the HIP backend (include/ps_hip.h, "layer-list models"): configuration, weight loading and the model object.
+
+A model directory holds config.json and model.safetensors.  config.json names the architecture; ARCHITECTURES maps it to the function that
+turns the configuration and the tensors into layer descriptors.  Every size and constant comes from config.json or a tensor's shape.
+
+Ranutar: a list of layers, each  x += norm_b(mixer(conv(norm(x))))  and, where it has one,  x += norm_b(ff(conv(norm(x)))), the mixer one of
+  wkv               per-channel decayed outer-product state with token-shift mixes and a bonus for the current token
+  delta             gated delta rule with short convolutions on q / k / v
+  latent_attention  attention over a low-rank latent + one shared rotated key part, sliding window
+the norms RMS with weights stored around zero, the feed-forward dense with the xIELU activation.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import json
+import os
+
+import numpy as np
+
+from . import hip
+from .safetensors_io import SafeTensors
+
+MIX_WKV, MIX_DELTA, MIX_LATENT = 1, 2, 3
+FF_NONE, FF_DENSE_XIELU = 0, 1
+
+
+class ConfigError(ValueError):
+    pass
+
+
+def _ranutar_layers(cfg: dict, st: SafeTensors, up) -> tuple[list, dict]:
+    """-> (list of hip.SeqLayer, top-level fields).  up.vec(array) / up.mat(bits) put a tensor on the device and return its handle."""
+    width = int(cfg["width"])
+    taps = int(cfg["canon"]["taps"])
+    layers = []
+    for i, lc in enumerate(cfg["layers"]):
+        p, mc, kind = f"l{i}.", lc["mixer"], lc["type"]
+        L = hip.SeqLayer()
+        for n in ("norm1", "norm1b"):
+            setattr(L, n, up.vec(st.f32(p + n)))
+        L.canon1 = up.vec(_expect(st, p + "canon1", (width, taps)))
+        mlp = lc.get("mlp")
+        if mlp:
+            if mlp.get("kind") != "dense":
+                raise ConfigError(f"layer {i}: feed-forward kind {mlp.get('kind')!r} is not known")
+            L.ff_kind, L.ff = FF_DENSE_XIELU, int(mlp["ff"])
+            for n in ("norm2", "norm2b"):
+                setattr(L, n, up.vec(st.f32(p + n)))
+            L.canon2 = up.vec(_expect(st, p + "canon2", (width, taps)))
+            act = st.f32(p + "mlp.act")
+            L.ff_act_p, L.ff_act_q = float(act[0]), float(act[1])
+            L.ff_up, L.ff_down = up.mat(st.bf16_bits(p + "mlp.up")), up.mat(st.bf16_bits(p + "mlp.down"))
+        m = p + "mix."
+        L.heads, L.dim = int(mc["heads"]), int(mc["dim"])
+        if kind == "wkv":
+            L.kind, L.vdim = MIX_WKV, L.dim
+            L.decay_rank = st.shape(m + "w1")[0]
+            L.in_r, L.in_k, L.in_v, L.in_g = (up.mat(st.bf16_bits(m + n)) for n in ("r", "k", "v", "g"))
+            L.decay1, L.decay2, L.out = up.mat(st.bf16_bits(m + "w1")), up.mat(st.bf16_bits(m + "w2")), up.mat(st.bf16_bits(m + "o"))
+            L.mu = up.vec(np.stack([st.f32(m + "mu." + n) for n in ("r", "k", "v", "g", "w")]))
+            L.decay0, L.bonus, L.onorm = up.vec(st.f32(m + "w0")), up.vec(st.f32(m + "u").reshape(-1)), up.vec(st.f32(m + "norm"))
+        elif kind == "delta":
+            L.kind, L.kv_heads, L.vdim, L.conv_taps = MIX_DELTA, int(mc["kv_heads"]), int(mc["vdim"]), int(mc["conv"])
+            L.in_cat = up.mat(np.concatenate([st.bf16_bits(m + n) for n in ("q", "k", "v", "g", "b", "a")], axis=0))
+            L.conv = up.vec(np.concatenate([_expect(st, m + n + ".conv", (st.shape(m + n)[0], L.conv_taps)) for n in ("q", "k", "v")], axis=0))
+            L.a_log, L.dt_bias, L.onorm = up.vec(st.f32(m + "A_log")), up.vec(st.f32(m + "dt_bias")), up.vec(st.f32(m + "norm"))
+            L.out = up.mat(st.bf16_bits(m + "o"))
+        elif kind == "latent_attention":
+            L.kind, L.vdim = MIX_LATENT, int(mc["vdim"])
+            L.q_rank, L.kv_rank, L.rot_dim = int(mc["q_rank"]), int(mc["kv_rank"]), int(mc["rot_dim"])
+            L.rot_dims, L.rot_base = int(mc["rot"]["dims"]), float(mc["rot"]["base"])
+            L.window, L.scale = int(mc["mask"]["size"]), float(mc["scale"])
+            L.in_cat = up.mat(np.concatenate([st.bf16_bits(m + "dq"), st.bf16_bits(m + "dkv")], axis=0))
+            L.uq = up.mat(st.bf16_bits(m + "uq"))
+            L.ukv = up.mat(np.concatenate([st.bf16_bits(m + "uk"), st.bf16_bits(m + "uv")], axis=0))
+            L.out = up.mat(st.bf16_bits(m + "o"))
+            L.qnorm, L.kvnorm = up.vec(st.f32(m + "dq.norm")), up.vec(st.f32(m + "dkv.norm"))
+        else:
+            raise ConfigError(f"layer {i}: mixer type {kind!r} is not known")
+        layers.append(L)
+    top = dict(width=width, vocab=int(cfg["vocab"]), canon_taps=taps, norm_eps=float(cfg["norm"]["eps"]), norm_offset=1.0,
+               logit_scale=float(cfg["logit_scale"]), embed=up.mat(st.bf16_bits("embed")), head=up.mat(st.bf16_bits("head")),
+               final_norm=up.vec(st.f32("final.norm")))
+    return layers, top
+
+
+def _expect(st: SafeTensors, name: str, shape: tuple) -> np.ndarray:
+    if st.shape(name) != tuple(shape):
+        raise ConfigError(f"tensor {name}: shape {st.shape(name)}, the configuration gives {tuple(shape)}")
+    return st.f32(name)
+
+
+ARCHITECTURES = {"Ranutar": _ranutar_layers}
+
+
+def read_config(model_dir: str) -> dict:
+    with open(os.path.join(model_dir, "config.json")) as f:
+        cfg = json.load(f)
+    if cfg.get("architecture") not in ARCHITECTURES:
+        raise ConfigError(f"unknown architecture {cfg.get('architecture')!r} (known: {sorted(ARCHITECTURES)})")
+    return cfg
+
+
+class _Uploader:
+    def __init__(self, ctx: hip.Ctx, as_f32: bool):
+        self.ctx, self.as_f32, self.vecs, self.mats = ctx, as_f32, [], []
+
+    def vec(self, a: np.ndarray) -> int:
+        d = self.ctx.to_device(np.ascontiguousarray(a, dtype=np.float32))
+        self.vecs.append(d)
+        return d.ptr
+
+    def mat(self, bits: np.ndarray) -> int:
+        bits = np.ascontiguousarray(bits, dtype=np.uint16)
+        h = C.c_void_p()
+        self.ctx.check(self.ctx.L.ps_hip_dense_upload(self.ctx.h, bits.ctypes.data_as(C.c_void_p), bits.shape[0], bits.shape[1], int(self.as_f32), C.byref(h)))
+        self.mats.append(h.value)
+        return h.value
+
+
+class SeqModel:
+    """ps_hip_seq over a model directory.  dtype "bfloat16": matrix products on bfloat16 operands, fp32 accumulation; "float32": fp32
+    throughout.  Sequences live in slots (acquire / release); forward() is the step function, generate() the greedy / sampled loop."""
+
+    def __init__(self, ctx: hip.Ctx, model_dir: str, dtype: str = "bfloat16", max_batch: int = 256, n_slots: int = 2):
+        if dtype not in ("bfloat16", "float32"):
+            raise ConfigError(f"dtype {dtype!r}: bfloat16 or float32")
+        self.ctx, self.dtype = ctx, dtype
+        self.cfg = read_config(model_dir)
+        self.arch = self.cfg["architecture"]
+        st = SafeTensors(os.path.join(model_dir, "model.safetensors"))
+        self._up = _Uploader(ctx, dtype == "float32")
+        layers, top = ARCHITECTURES[self.arch](self.cfg, st, self._up)
+        self._layers = (hip.SeqLayer * len(layers))(*layers)
+        d = hip.SeqDesc()
+        d.n_layers, d.max_batch, d.n_slots, d.compute = len(layers), int(max_batch), int(n_slots), int(dtype == "float32")
+        for k, v in top.items():
+            setattr(d, k, v)
+        d.layers = self._layers
+        self.vocab, self.width, self.n_layers, self.max_batch = d.vocab, d.width, d.n_layers, int(max_batch)
+        h = C.c_void_p()
+        ctx.check(ctx.L.ps_hip_seq_create(ctx.h, C.byref(d), C.byref(h)))
+        self.h = h
+        self._dbg = None
+
+    def close(self):
+        if getattr(self, "h", None):
+            self.ctx.L.ps_hip_seq_destroy(self.h)
+            self.h = None
+            for m in self._up.mats:
+                self.ctx.L.ps_hip_dense_free(self.ctx.h, m)
+            for v in self._up.vecs:
+                v.free()
+            if self._dbg is not None:
+                self._dbg.free()
+
+    # ---- state manager
+    def acquire(self) -> int:
+        s = C.c_int(-1)
+        self.ctx.check(self.ctx.L.ps_hip_seq_acquire(self.h, C.byref(s)))
+        return s.value
+
+    def release(self, slot: int):
+        self.ctx.check(self.ctx.L.ps_hip_seq_release(self.h, int(slot)))
+
+    def position(self, slot: int) -> int:
+        return int(self.ctx.L.ps_hip_seq_position(self.h, int(slot)))
+
+    @property
+    def slot_bytes(self) -> int:
+        return int(self.ctx.L.ps_hip_seq_slot_bytes(self.h))
+
+    @property
+    def weight_bytes_per_token(self) -> int:
+        return int(self.ctx.L.ps_hip_seq_weight_bytes_per_token(self.h))
+
+    def set_mode(self, mode: int):
+        self.ctx.L.ps_hip_seq_set_mode(self.h, int(mode))
+
+    # ---- step function
+    def forward(self, slot: int, tokens, want=None, argmax: bool = False):
+        """The next tokens of the sequence in `slot`; want: ascending indices into them.  -> logits [len(want), vocab] (or their arg-max ids)."""
+        tokens = np.ascontiguousarray(tokens, dtype=np.int32)
+        want = np.ascontiguousarray(want if want is not None else [], dtype=np.int32)
+        out = np.empty((want.size, self.vocab), dtype=np.float32) if not argmax else None
+        ids = np.empty(want.size, dtype=np.int32) if argmax else None
+        self.ctx.check(self.ctx.L.ps_hip_seq_forward(self.h, int(slot), hip._ptr(tokens), tokens.size, hip._ptr(want) if want.size else None, want.size,
+                                                     hip._ptr(out) if out is not None and want.size else None, hip._ptr(ids) if ids is not None and want.size else None))
+        return ids if argmax else out
+
+    def decode_greedy(self, slot: int, token: int, steps: int) -> np.ndarray:
+        out = np.empty(steps, dtype=np.int32)
+        self.ctx.check(self.ctx.L.ps_hip_seq_decode_greedy(self.h, int(slot), int(token), int(steps), hip._ptr(out)))
+        return out
+
+    def generate(self, prompt, steps: int, sampler=None) -> np.ndarray:
+        """Prefill all but the last prompt token without logits, then `steps` tokens: greedy on the device (sampler None), or each step's logits
+        through `sampler` (a callable logits -> token id, e.g. host.Sampler.sample)."""
+        prompt = np.ascontiguousarray(prompt, dtype=np.int32)
+        slot = self.acquire()
+        try:
+            if prompt.size > 1:
+                self.forward(slot, prompt[:-1])
+            if sampler is None:
+                return self.decode_greedy(slot, int(prompt[-1]), steps)
+            out, tok = [], int(prompt[-1])
+            for _ in range(steps):
+                tok = int(sampler(self.forward(slot, [tok], want=[0])[0]))
+                out.append(tok)
+            return np.asarray(out, dtype=np.int32)
+        finally:
+            self.release(slot)
+
+    # ---- diagnostics
+    def capture_layers(self, on: bool = True):
+        """Keep the residual stream after every layer of the next forwards (each at most max_batch tokens)."""
+        if on and self._dbg is None:
+            self._dbg = self.ctx.empty((self.n_layers, self.max_batch, self.width), np.float32)
+        self.ctx.check(self.ctx.L.ps_hip_seq_debug_layers(self.h, self._dbg.ptr if on else None))
+
+    def layers(self, n_tokens: int) -> np.ndarray:
+        self.ctx.sync()
+        return self._dbg.numpy()[:, :n_tokens]
+
+
+def is_seq_model_dir(model_dir: str) -> bool:
+    return os.path.exists(os.path.join(model_dir, "config.json")) and os.path.exists(os.path.join(model_dir, "model.safetensors"))
+
+
+def load_model(ctx: hip.Ctx, model_dir: str, **kw):
+    """The registry's front door: config.json + model.safetensors -> SeqModel (by its architecture), model.json + ggml/weights.gguf -> hip.Model."""
+    if is_seq_model_dir(model_dir):
+        return SeqModel(ctx, model_dir, **kw)
+    if os.path.exists(os.path.join(model_dir, "model.json")):
+        kw.pop("dtype", None)
+        kw.pop("n_slots", None)
+        return hip.Model(ctx, model_dir, **kw)
+    raise ConfigError(f"{model_dir}: neither config.json + model.safetensors nor model.json + ggml/weights.gguf")
+
+
+class RequestScheduler:
+    """Requests by id over a model's slots: a request's first tokens take a slot, later portions continue it, finish() gives the slot back.
+    Requests are served one portion at a time in the order they are handed in."""
+
+    def __init__(self, model: SeqModel):
+        self.model, self.slots = model, {}
+
+    def feed(self, rid, tokens, want=None) -> np.ndarray:
+        if rid not in self.slots:
+            self.slots[rid] = self.model.acquire()
+        return self.model.forward(self.slots[rid], tokens, want)
+
+    def finish(self, rid):
+        s = self.slots.pop(rid, None)
+        if s is not None:
+            self.model.release(s)
+
+    def live_tokens(self) -> int:
+        return sum(self.model.position(s) for s in self.slots.values())
