@@ -215,3 +215,78 @@ def truncate_model_dir(src_dir: str, out_dir: str, n_layers: int, model_id: str 
 def load_model_json(model_dir: str) -> dict:
     with open(os.path.join(model_dir, "model.json")) as f:
         return json.load(f)
+
+
+# ---------------------------------------------------------------------------------------------------- layer-list models (config.json + model.safetensors)
+def seq_layer(kind: str, ff: int | None = 64, **mixer) -> dict:
+    """One entry of a layer-list configuration's 'layers'."""
+    return {"type": kind, "mixer": dict(mixer), "mlp": {"ff": int(ff), "kind": "dense"} if ff else None}
+
+
+def seq_config(width: int, vocab: int, layers: list, taps: int = 3, eps: float = 1e-6, logit_scale: float = 1.0, architecture: str = "Ranutar") -> dict:
+    return {"architecture": architecture, "canon": {"taps": int(taps)}, "layers": layers, "logit_scale": float(logit_scale), "norm": {"eps": float(eps)},
+            "vocab": int(vocab), "width": int(width)}
+
+
+def seq_tensors(cfg: dict, seed: int = 0, decay_rank: int = 8) -> dict:
+    """Random-init tensors of a layer-list configuration, name -> float32 array already rounded to bfloat16 (what the file will hold)."""
+    from .safetensors_io import f32_to_bf16_bits
+    rng = np.random.default_rng(seed)
+    W, taps = cfg["width"], cfg["canon"]["taps"]
+    t = {}
+
+    def lin(n, k, gain=1.0):
+        return rng.standard_normal((n, k), dtype=np.float32) * np.float32(gain / np.sqrt(k))
+
+    def vec(n, std=0.1, mean=0.0):
+        return (rng.standard_normal(n, dtype=np.float32) * np.float32(std) + np.float32(mean)).astype(np.float32)
+
+    t["embed"] = rng.standard_normal((cfg["vocab"], W), dtype=np.float32)
+    for i, lc in enumerate(cfg["layers"]):
+        p, m, mc = f"l{i}.", f"l{i}.mix.", lc["mixer"]
+        for n in ("norm1", "norm1b"):
+            t[p + n] = vec(W)
+        t[p + "canon1"] = (rng.standard_normal((W, taps), dtype=np.float32) * np.float32(0.3)).astype(np.float32)
+        if lc.get("mlp"):
+            ff = lc["mlp"]["ff"]
+            for n in ("norm2", "norm2b"):
+                t[p + n] = vec(W)
+            t[p + "canon2"] = (rng.standard_normal((W, taps), dtype=np.float32) * np.float32(0.3)).astype(np.float32)
+            t[p + "mlp.up"], t[p + "mlp.down"], t[p + "mlp.act"] = lin(ff, W), lin(W, ff), vec(2, 0.7)
+        H, d = mc["heads"], mc["dim"]
+        if lc["type"] == "wkv":
+            for n in ("r", "k", "v", "g", "w"):
+                t[m + "mu." + n] = rng.random(W, dtype=np.float32)
+            for n in ("r", "k", "v", "g"):
+                t[m + n] = lin(H * d, W)
+            t[m + "w1"], t[m + "w2"], t[m + "w0"] = lin(decay_rank, W), lin(H * d, decay_rank), vec(H * d, 0.8, -0.5)
+            t[m + "u"] = rng.standard_normal((H, d), dtype=np.float32) * np.float32(0.5)
+            t[m + "norm"], t[m + "o"] = vec(H * d, 0.2, 1.0), lin(W, H * d)
+        elif lc["type"] == "delta":
+            KH, dv, ct = mc["kv_heads"], mc["vdim"], mc["conv"]
+            for n, rows in (("q", KH * d), ("k", KH * d), ("v", H * dv)):
+                t[m + n] = lin(rows, W)
+                t[m + n + ".conv"] = (rng.standard_normal((rows, ct), dtype=np.float32) * np.float32(0.6)).astype(np.float32)
+            t[m + "b"], t[m + "a"], t[m + "g"], t[m + "o"] = lin(H, W), lin(H, W), lin(H * dv, W), lin(W, H * dv)
+            t[m + "A_log"] = np.log(rng.uniform(0.5, 4.0, H)).astype(np.float32)
+            t[m + "dt_bias"], t[m + "norm"] = vec(H, 0.5), vec(dv, 0.2, 1.0)
+        elif lc["type"] == "latent_attention":
+            dv, qr, kr, dr = mc["vdim"], mc["q_rank"], mc["kv_rank"], mc["rot_dim"]
+            t[m + "dq"], t[m + "dq.norm"], t[m + "uq"] = lin(qr, W), vec(qr, 0.2, 1.0), lin(H * (d + dr), qr)
+            t[m + "dkv"], t[m + "dkv.norm"] = lin(kr + dr, W), vec(kr, 0.2, 1.0)
+            t[m + "uk"], t[m + "uv"], t[m + "o"] = lin(H * d, kr), lin(H * dv, kr), lin(W, H * dv)
+        else:
+            raise ValueError(lc["type"])
+    t["final.norm"], t["head"] = vec(W), lin(cfg["vocab"], W)
+    return {k: (f32_to_bf16_bits(v).astype(np.uint32) << 16).view(np.float32).reshape(v.shape) for k, v in t.items()}
+
+
+def write_seq_model_dir(out_dir: str, cfg: dict, seed: int = 0, tensors: dict | None = None) -> dict:
+    """config.json + model.safetensors (bfloat16) of a layer-list model; returns the tensors as the file holds them (float32 views)."""
+    from . import safetensors_io
+    os.makedirs(out_dir, exist_ok=True)
+    tensors = tensors if tensors is not None else seq_tensors(cfg, seed)
+    with open(os.path.join(out_dir, "config.json"), "w") as f:
+        json.dump(cfg, f, indent=1)
+    safetensors_io.write(os.path.join(out_dir, "model.safetensors"), tensors)
+    return tensors
