@@ -52,6 +52,9 @@ def parse():
     ap.add_argument("--cpu-reference-limit", type=int, default=150, help="seconds the reference CPU baseline (a child process) may take before it is killed")
     ap.add_argument("--cpu-reference-child", default=None, help=argparse.SUPPRESS)
     ap.add_argument("--f16-super-chunk", type=int, default=2048, help="side leg (fp16 perf mode): tokens per mat-mul launch")
+    ap.add_argument("--layer-list", default=None, metavar="SIZES", help="instead of the headline workload: prefill / decode throughput of a layer-list model (dense bf16 "
+                    "matrices; powerserve_amd/bench_seq.py SIZES, comma-separated, or 'all') beside the Q4_K Llama path at equal width")
+    ap.add_argument("--layer-list-portion", type=int, default=512, help="--layer-list: tokens per launch sequence of the prefill")
     ap.add_argument("--prefill-warmup-tokens", type=int, default=128, help="untimed tokens forwarded before the timed prefill (first use of the prefill kernels in the process; 0: none)")
     ap.add_argument("--wide-chunk", type=int, default=512, help="side leg: prefill in chunks of this many tokens (0: skip)")
     ap.add_argument("--super-chunks", type=int, default=4, help="reference-sized prefill chunks (--batch tokens each) per launch sequence "
@@ -419,6 +422,12 @@ def main():
     args = parse()
     if args.cpu_reference_child:  # (the guarded baseline's child process: CPU only, one JSON line)
         _cpu_reference_child(args.cpu_reference_child)
+        return
+    if args.layer_list:  # a side workload with its own record; the default workload and its contract are untouched
+        from powerserve_amd import bench_seq
+        names = list(bench_seq.SIZES) if args.layer_list == "all" else args.layer_list.split(",")
+        steps = args.steps if args.steps != 256 else 64
+        print(json.dumps(bench_seq.run(names, prompt_len=args.prompt_len, steps=steps, max_batch=args.layer_list_portion)), flush=True)
         return
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         relaunch_distributed(args)  # does not return

@@ -378,9 +378,9 @@ int ps_hip_seq_debug_layers(ps_hip_seq *m, float *buf_dev);
  * wherever a faster form exists (per-key attention, tiled mat-mul for single tokens) -- same results up to rounding */
 int ps_hip_seq_set_mode(ps_hip_seq *m, int mode);
 uint64_t ps_hip_seq_weight_bytes_per_token(const ps_hip_seq *m);
-/* Measurement helper: one kernel family of the step function replayed `reps` times on the model's own buffers between
- * HIP events -> microseconds per launch and the bytes / flops it moves (bench.py's per-kernel roofline).
- * which: 0 feed-forward up mat-vec (single token), 1 the same for T tokens, 2 wkv scan, 3 delta scan, 4 latent attention */
+/* Measurement helper (bench.py's per-kernel roofline): a feed-forward matrix product of T tokens replayed `reps` times over every layer
+ * that has one (each launch streams its own layer's weights), between HIP events -> microseconds per launch, the weight bytes and the
+ * flops of one launch.  which: 0 the up projection (with its activation), 1 the down projection.  T <= 8 runs the mat-vec. */
 int ps_hip_seq_bench_kernel(ps_hip_seq *m, int which, int T, int reps, double *us_per_launch, double *bytes, double *flops);
 
 #ifdef __cplusplus

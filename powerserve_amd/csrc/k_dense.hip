@@ -192,29 +192,37 @@ __global__ __launch_bounds__(256) void dense_mv_kernel(dn_args g) {
 #pragma unroll
             for (int c = 0; c < C; c++) acc[r][c] = 0.f;
         if (vec) {
-            for (long long k = (long long)lane * VE; k < K; k += 64 * VE) {
-                dn_f4 raw[RW];
+            // two 16-byte pieces of each of the four rows in flight per lane (8 KiB per wave and round)
+            for (long long k = (long long)lane * VE; k < K; k += 128 * VE) {
+                const long long k2 = k + 64 * VE;
+                const bool two = k2 < K;
+                dn_f4 raw[2][RW];
 #pragma unroll
                 for (int r = 0; r < RW; r++) {
                     const long long n = nb + r < g.N ? nb + r : g.N - 1;
-                    raw[r] = __builtin_nontemporal_load((const dn_f4 *)(W + n * K + k));
+                    raw[0][r] = __builtin_nontemporal_load((const dn_f4 *)(W + n * K + k));
+                    raw[1][r] = two ? __builtin_nontemporal_load((const dn_f4 *)(W + n * K + k2)) : dn_f4{0.f, 0.f, 0.f, 0.f};
                 }
 #pragma unroll
-                for (int r = 0; r < RW; r++) {
-                    float wv[VE];
-                    if constexpr (sizeof(WT) == 2) {
-                        unsigned short h[8];
-                        __builtin_memcpy(h, &raw[r], 16);
+                for (int u = 0; u < 2; u++) {
+                    const long long ku = u ? (two ? k2 : k) : k; // (the second piece is zero where there is none: any valid x offset will do)
 #pragma unroll
-                        for (int e = 0; e < 8; e++) wv[e] = dn_bf2f(h[e]);
-                    } else {
-                        __builtin_memcpy(wv, &raw[r], 16);
-                    }
+                    for (int r = 0; r < RW; r++) {
+                        float wv[VE];
+                        if constexpr (sizeof(WT) == 2) {
+                            unsigned short h[8];
+                            __builtin_memcpy(h, &raw[u][r], 16);
 #pragma unroll
-                    for (int c = 0; c < C; c++) {
-                        const float *x = xs + (long long)c * Kp + k;
+                            for (int e = 0; e < 8; e++) wv[e] = dn_bf2f(h[e]);
+                        } else {
+                            __builtin_memcpy(wv, &raw[u][r], 16);
+                        }
 #pragma unroll
-                        for (int e = 0; e < VE; e++) acc[r][c] = fmaf(wv[e], x[e], acc[r][c]);
+                        for (int c = 0; c < C; c++) {
+                            const float *x = xs + (long long)c * Kp + ku;
+#pragma unroll
+                            for (int e = 0; e < VE; e++) acc[r][c] = fmaf(wv[e], x[e], acc[r][c]);
+                        }
                     }
                 }
             }
@@ -240,6 +248,97 @@ __global__ __launch_bounds__(256) void dense_mv_kernel(dn_args g) {
                 if (lane == 0 && nb + r < g.N && c < T) g.out[(long long)c * g.ldo + nb + r] = dn_epi(g, v, nb + r);
             }
     }
+}
+
+
+// ---------------------------------------------------------------------------------------------------- wide mat-mul (bf16, K % 64 == 0)
+// The A operand is first packed to bfloat16 [Tp][K] (Tp = T rounded up to 128, rows beyond T zero; the ring rows and the token-shift mix
+// are resolved there), then 128 tokens x 128 outputs per work-group: four waves of 64 x 64 (4 x 4 tiles of v_mfma_f32_16x16x32_bf16), K in
+// steps of 64 through LDS (rows padded to 144 B), the next step's 16-byte global loads in flight while the matrix cores run the current one.
+__global__ __launch_bounds__(256) void dense_pack_kernel(dn_args g, unsigned short *out, int Tp) {
+    long long row0;
+    int T;
+    dn_rows(g, row0, T);
+    const long long per_row = g.K / 8, total = (long long)Tp * per_row;
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long long)gridDim.x * 256) {
+        const int t = (int)(i / per_row);
+        const long long k = (i % per_row) * 8;
+        dn_us8 v;
+#pragma unroll
+        for (int e = 0; e < 8; e++) v[e] = t < T ? dn_f2bf(dn_aval(g, row0, t, k + e)) : (unsigned short)0;
+        *(dn_us8 *)(out + (long long)t * g.K + k) = v;
+    }
+}
+
+#define DN_FLD 72 // LDS row stride in bf16: 64 + 8
+__global__ __launch_bounds__(256) void dense_mm_fast_kernel(dn_args g, const unsigned short *A) {
+    __shared__ __attribute__((aligned(16))) unsigned short As[128 * DN_FLD];
+    __shared__ __attribute__((aligned(16))) unsigned short Bs[128 * DN_FLD];
+    long long row0;
+    int T;
+    dn_rows(g, row0, T);
+    const int t0 = blockIdx.y * 128;
+    if (t0 >= T) return;
+    const long long n0 = (long long)blockIdx.x * 128;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1, lr = lane & 15, lq = lane >> 4;
+    const unsigned short *W = (const unsigned short *)g.w;
+    const long long K = g.K;
+    // staging: 128 rows x 64 k = 1024 pieces of 16 bytes per operand, four per thread: row = (tid >> 3) + 32 i, k piece = tid & 7
+    const int sr = tid >> 3, sk = (tid & 7) * 8;
+    const unsigned short *ap[4], *bp[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        ap[i] = A + (long long)(t0 + sr + 32 * i) * K + sk; // (the packed operand has Tp rows: always there)
+        long long n = n0 + sr + 32 * i;
+        if (n >= g.N) n = g.N - 1;
+        bp[i] = W + n * K + sk;
+    }
+    dn_f4 ra[4], rb[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) { ra[i] = *(const dn_f4 *)ap[i]; rb[i] = *(const dn_f4 *)bp[i]; }
+    dn_f4 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = dn_f4{0.f, 0.f, 0.f, 0.f};
+    for (long long k0 = 0; k0 < K; k0 += 64) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            *(dn_f4 *)&As[(sr + 32 * i) * DN_FLD + sk] = ra[i];
+            *(dn_f4 *)&Bs[(sr + 32 * i) * DN_FLD + sk] = rb[i];
+        }
+        __syncthreads();
+        if (k0 + 64 < K) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) { ra[i] = *(const dn_f4 *)(ap[i] + k0 + 64); rb[i] = *(const dn_f4 *)(bp[i] + k0 + 64); }
+        }
+#pragma unroll
+        for (int kk = 0; kk < 64; kk += 32) {
+            dn_bf8 fa[4], fb[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const dn_f4 xa = *(const dn_f4 *)&As[(wm * 64 + i * 16 + lr) * DN_FLD + kk + lq * 8];
+                const dn_f4 xb = *(const dn_f4 *)&Bs[(wn * 64 + i * 16 + lr) * DN_FLD + kk + lq * 8];
+                __builtin_memcpy(&fa[i], &xa, 16);
+                __builtin_memcpy(&fb[i], &xb, 16);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int t = t0 + wm * 64 + i * 16 + lq * 4 + e;
+                const long long n = n0 + wn * 64 + j * 16 + lr;
+                if (t < T && n < g.N) g.out[(long long)t * g.ldo + n] = dn_epi(g, acc[i][j][e], n);
+            }
 }
 
 template <typename WT, int C>
@@ -276,6 +375,14 @@ int psk_dense(hipStream_t st, const psk_dense_args &a) {
             }
             return 0;
         }
+    }
+    const int Tp = (a.T + 127) / 128 * 128;
+    if (bf && !a.force_tiled && a.T > 8 && g.K % 64 == 0 && a.pack && (size_t)Tp * g.K * 2 <= a.pack_bytes) {
+        long long pb = ((long long)Tp * (g.K / 8) + 255) / 256;
+        if (pb > 8192) pb = 8192;
+        hipLaunchKernelGGL(dense_pack_kernel, dim3((unsigned)pb), dim3(256), 0, st, g, (unsigned short *)a.pack, Tp);
+        hipLaunchKernelGGL(dense_mm_fast_kernel, dim3((unsigned)((g.N + 127) / 128), (unsigned)(Tp / 128)), dim3(256), 0, st, g, (const unsigned short *)a.pack);
+        return 0;
     }
     dim3 grid((unsigned)((g.N + 63) / 64), (unsigned)((a.T + 63) / 64));
     if (bf) hipLaunchKernelGGL(dense_mm_kernel<unsigned short>, grid, dim3(256), 0, st, g);

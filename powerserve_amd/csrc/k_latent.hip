@@ -118,3 +118,306 @@ void psk_latent_attn(hipStream_t st, const ps_seq_step *step, int64_t ring_off, 
     hipLaunchKernelGGL(latent_attn_kernel, dim3(T, H), dim3(64), (size_t)(d + dr + 64) * 4, st, step, (long long)ring_off, cap, q, (long long)ldq, kv, (long long)ldkv,
                        freq, H, d, dr, rot_dims, dv, kv_rank, window, scale, o, (long long)ldo);
 }
+
+// ---------------------------------------------------------------------------------------------------- matrix-core form
+// One wave attends 16 rows to tiles of 16 keys, fp32 throughout on v_mfma_f32_16x16x4_f32:
+//   scores   S[16 x 16] = Q[16 x DK] K^T: the keys come straight from memory as 16-byte pieces (lane (key l % 16, quarter l / 16) holds 4
+//            consecutive dimensions; the row operand is read from LDS in the same order, so the sum runs over a permutation of the dimensions)
+//   soft-max online, in the accumulator layout (lane holds rows 4 (l / 16) + i of key column l % 16; a row's 16 lanes reduce by butterfly)
+//   output   O[16 x DV] += P V: P goes through a 16 x 17 LDS patch into the row-operand layout; V comes as 16-byte pieces of 4 consecutive
+//            columns, so accumulator tile jj of a 64-column group holds columns 4 (l % 16) + jj -- undone at the final store.
+// A "row" is a (token, head) pair.  Two drivers use it: a prompt's portion over per-head keys / values expanded from the ring (rows = 16
+// consecutive tokens of one head), and the single-token step in the ABSORBED form -- rows = heads, every head's query folded through its key
+// expansion into latent space (q~_h = W_uk,h^T q_h), keys AND values the ring's latents themselves, the value expansion applied afterwards to
+// the attended latent -- where the ring is read once for all heads and nothing is expanded per key.
+typedef float la_f4 __attribute__((ext_vector_type(4)));
+
+struct la_src { // where key j's row lives: base + ((j - sub) mod `mod`) * ld   (mod 0: no wrap)
+    const float *base;
+    long long ld, sub, mod;
+};
+static __device__ __forceinline__ const float *la_row(const la_src &s, long long j) {
+    long long r = j - s.sub;
+    if (s.mod > 0) r %= s.mod;
+    return s.base + r * s.ld;
+}
+
+// qs: this wave's 16 rows in LDS, row stride qld floats, [DK1 | DK2]; pt: its 16 x 17 patch.  rowpos(i): position of accumulator row i of this
+// lane (rows 4 (l / 16) + i), < 0 for a row that does not exist.  Keys j0 .. j0 + 15 are visible to a row at position p when j <= p, j > p - window
+// and j < jend.  NJ: accumulator tiles (DV <= 16 NJ).
+template <int NJ>
+static __device__ __forceinline__ void la_tile(const float *qs, int qld, float *pt, const la_src &k1, const la_src &k2, const la_src &vs, int DK1, int DK2, int DV,
+                                               long long j0, long long jend, const long long (&rowpos)[4], int window, float scale, float (&m)[4], float (&l)[4],
+                                               la_f4 (&acc)[NJ]) {
+    const int lane = threadIdx.x & 63, lr = lane & 15, lq = lane >> 4;
+    const long long jk = j0 + lr < jend ? j0 + lr : jend - 1; // (a key row that exists; masked below)
+    la_f4 s4 = {0.f, 0.f, 0.f, 0.f};
+    const float *kr1 = la_row(k1, jk) + 4 * lq, *kr2 = la_row(k2, jk) + 4 * lq, *qr = qs + lr * qld + 4 * lq;
+    for (int g = 0; g < DK1; g += 16) {
+        const la_f4 b = *(const la_f4 *)(kr1 + g), a = *(const la_f4 *)(qr + g);
+#pragma unroll
+        for (int e = 0; e < 4; e++) s4 = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], b[e], s4, 0, 0, 0);
+    }
+    for (int g = 0; g < DK2; g += 16) {
+        const la_f4 b = *(const la_f4 *)(kr2 + g), a = *(const la_f4 *)(qr + DK1 + g);
+#pragma unroll
+        for (int e = 0; e < 4; e++) s4 = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], b[e], s4, 0, 0, 0);
+    }
+    const long long j = j0 + lr;
+    float p[4], corr[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const bool vis = rowpos[i] >= 0 && j < jend && j <= rowpos[i] && j > rowpos[i] - window;
+        const float s = vis ? s4[i] * scale : -INFINITY;
+        float tm = s;
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) tm = fmaxf(tm, __shfl_xor(tm, o, 64));
+        const float mn = fmaxf(m[i], tm);
+        corr[i] = mn == -INFINITY ? 1.f : expf(m[i] - mn);
+        p[i] = mn == -INFINITY ? 0.f : expf(s - mn);
+        float ts = p[i];
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) ts += __shfl_xor(ts, o, 64);
+        l[i] = l[i] * corr[i] + ts;
+        m[i] = mn;
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int i = 0; i < 4; i++) pt[(4 * lq + i) * 17 + lr] = p[i];
+    __builtin_amdgcn_wave_barrier();
+    float pa[4];
+#pragma unroll
+    for (int s = 0; s < 4; s++) pa[s] = pt[lr * 17 + 4 * s + lq];
+    __builtin_amdgcn_wave_barrier();
+    const float *vr[4];
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        const long long jv = j0 + 4 * s + lq < jend ? j0 + 4 * s + lq : jend - 1; // (weight 0 beyond the end)
+        vr[s] = la_row(vs, jv) + 4 * lr;
+    }
+#pragma unroll
+    for (int J = 0; J < NJ / 4; J++) {
+        if (64 * J < DV) {
+            const bool in = 64 * J + 4 * lr < DV;
+            la_f4 b[4];
+#pragma unroll
+            for (int s = 0; s < 4; s++) b[s] = in ? *(const la_f4 *)(vr[s] + 64 * J) : la_f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++) {
+                la_f4 a = acc[4 * J + jj];
+#pragma unroll
+                for (int i = 0; i < 4; i++) a[i] *= corr[i];
+#pragma unroll
+                for (int s = 0; s < 4; s++) a = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[s], b[s][jj], a, 0, 0, 0);
+                acc[4 * J + jj] = a;
+            }
+        }
+    }
+}
+
+// a prompt's portion: block = 64 consecutive tokens of one head (a wave per 16), keys / values expanded per head in kv (position first + row)
+// dynamic LDS: 4 x (16 x qld + 16 x 17)
+template <int NJ>
+__global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const ps_seq_step *step, long long ring_off, int cap, const float *q, long long ldq, const float *kv,
+                                                               long long ldkv, const float *freq, int H, int d, int dr, int rot_dims, int dv, int kv_rank, int window,
+                                                               float scale, int T, float *o, long long ldo) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lq = lane >> 4, h = blockIdx.y;
+    const int qld = d + dr + 4;
+    float *qs = lds + wave * (16 * qld + 16 * 17), *pt = qs + 16 * qld;
+    const long long pos0 = step->pos0;
+    const int t0 = blockIdx.x * 64 + wave * 16;
+    if (t0 >= T) return; // (no block-wide barrier below: waves are on their own)
+    const long long first = pos0 - window + 1 > 0 ? pos0 - window + 1 : 0;
+    const int half = rot_dims / 2;
+    for (int x = lane; x < 16 * (d + dr); x += 64) {
+        const int r = x / (d + dr), c = x % (d + dr), t = t0 + r;
+        float v = 0.f;
+        if (t < T) {
+            const float *qt = q + (long long)t * ldq + (long long)h * (d + dr);
+            v = qt[c];
+            const int cr = c - d;
+            if (cr >= 0 && cr < 2 * half) {
+                const int i = cr < half ? cr : cr - half;
+                const float ang = (float)(pos0 + t) * freq[i], cs = cosf(ang), sn = sinf(ang);
+                v = cr < half ? qt[d + i] * cs - qt[d + half + i] * sn : qt[d + half + i] * cs + qt[d + i] * sn;
+            }
+        }
+        qs[r * qld + c] = v;
+    }
+    __builtin_amdgcn_wave_barrier();
+    const la_src k1 = {kv + (long long)h * d, ldkv, first, 0};
+    const la_src k2 = {step->state + ring_off + kv_rank, (long long)(kv_rank + dr), 0, cap};
+    const la_src vs = {kv + (long long)H * d + (long long)h * dv, ldkv, first, 0};
+    long long rowpos[4];
+    float m[4], l[4];
+    la_f4 acc[NJ];
+#pragma unroll
+    for (int i = 0; i < 4; i++) { rowpos[i] = t0 + 4 * lq + i < T ? pos0 + t0 + 4 * lq + i : -1; m[i] = -INFINITY; l[i] = 0.f; }
+#pragma unroll
+    for (int j = 0; j < NJ; j++) acc[j] = la_f4{0.f, 0.f, 0.f, 0.f};
+    const long long plast = pos0 + (t0 + 15 < T ? t0 + 15 : T - 1), pfirst = pos0 + t0;
+    const long long lo = pfirst - window + 1 > 0 ? pfirst - window + 1 : 0;
+    for (long long j0 = lo; j0 <= plast; j0 += 16) la_tile<NJ>(qs, qld, pt, k1, k2, vs, d, dr, dv, j0, plast + 1, rowpos, window, scale, m, l, acc);
+#pragma unroll
+    for (int J = 0; J < NJ / 4; J++)
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int t = t0 + 4 * lq + i, c = 64 * J + 4 * lr + jj;
+                if (t < T && c < dv) o[(long long)t * ldo + (long long)h * dv + c] = acc[4 * J + jj][i] / l[i];
+            }
+}
+
+bool psk_latent_attn_mfma_ok(int d, int dr, int dv) { return d % 16 == 0 && dr % 16 == 0 && dv % 4 == 0 && dv <= 128 && (size_t)4 * (16 * (d + dr + 4) + 16 * 17) * 4 <= 160 * 1024; }
+void psk_latent_attn_mfma(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, const float *q, int64_t ldq, const float *kv, int64_t ldkv,
+                          const float *freq, int H, int d, int dr, int rot_dims, int dv, int kv_rank, int window, float scale, int T, float *o, int64_t ldo) {
+    const size_t lds = (size_t)4 * (16 * (d + dr + 4) + 16 * 17) * 4;
+    static unsigned long long mask = 0;
+    if (ps_first_on_device(&mask)) (void)hipFuncSetAttribute((const void *)latent_attn_mfma_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    hipLaunchKernelGGL(latent_attn_mfma_kernel<8>, dim3((T + 63) / 64, H), dim3(256), lds, st, step, (long long)ring_off, cap, q, (long long)ldq, kv, (long long)ldkv, freq,
+                       H, d, dr, rot_dims, dv, kv_rank, window, scale, T, o, (long long)ldo);
+}
+
+// ---------------------------------------------------------------------------------------------------- single token, absorbed
+// qa[h][r] = sum_i q[h][i] Wuk[h * d + i][r]: a head's query folded into latent space.  One block per head, a thread per latent index.
+template <typename WT>
+__global__ __launch_bounds__(256) void latent_fold_q_kernel(const float *q, int qstride, const WT *wuk, int d, int R, float *qa) {
+    const int h = blockIdx.x;
+    const float *qh = q + (long long)h * qstride;
+    for (int r = threadIdx.x; r < R; r += 256) {
+        float a = 0.f;
+        for (int i = 0; i < d; i++) {
+            float w;
+            if constexpr (sizeof(WT) == 2) w = __uint_as_float((unsigned)wuk[((long long)h * d + i) * R + r] << 16);
+            else w = wuk[((long long)h * d + i) * R + r];
+            a = fmaf(qh[i], w, a);
+        }
+        qa[(long long)h * R + r] = a;
+    }
+}
+// o[h][x] = sum_r Wuv[h * dv + x][r] ol[h][r]: the value expansion of the attended latent.  A wave per output row.
+template <typename WT>
+__global__ __launch_bounds__(256) void latent_unfold_v_kernel(const float *ol, const WT *wuv, int dv, int R, int rows, float *o) {
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (row >= rows) return;
+    const float *x = ol + (long long)(row / dv) * R;
+    float a = 0.f;
+    for (int r = lane; r < R; r += 64) {
+        float w;
+        if constexpr (sizeof(WT) == 2) w = __uint_as_float((unsigned)wuv[(long long)row * R + r] << 16);
+        else w = wuv[(long long)row * R + r];
+        a = fmaf(w, x[r], a);
+    }
+    a = la_wave_sum(a);
+    if (lane == 0) o[row] = a;
+}
+
+// rows = heads (16 per block), keys = ring rows; wave w of block (split s, head tile) takes key tile 4 s + w of the window.  Partials
+// part[(tile * H16 + ht) ...]: per (key tile, head) m, l and R unnormalised outputs.  dynamic LDS: 16 x qld + 4 x 16 x 17
+template <int NJ>
+__global__ __launch_bounds__(256) void latent_absorbed_kernel(const ps_seq_step *step, long long ring_off, int cap, const float *qa, const float *q, int qstride, int d,
+                                                              int dr, int rot_dims, const float *freq, int H, int R, int window, float scale, float *part) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lq = lane >> 4, h0 = blockIdx.y * 16;
+    const int qld = R + dr + 4;
+    float *qs = lds, *pt = lds + 16 * qld + wave * 16 * 17;
+    const long long p = step->pos0;
+    const long long lo = p - window + 1 > 0 ? p - window + 1 : 0;
+    const int half = rot_dims / 2;
+    for (int x = threadIdx.x; x < 16 * (R + dr); x += 256) {
+        const int r = x / (R + dr), c = x % (R + dr), h = h0 + r;
+        float v = 0.f;
+        if (h < H) {
+            if (c < R) v = qa[(long long)h * R + c];
+            else {
+                const float *qt = q + (long long)h * qstride + d;
+                const int cr = c - R;
+                v = qt[cr];
+                if (cr < 2 * half) {
+                    const int i = cr < half ? cr : cr - half;
+                    const float ang = (float)p * freq[i], cs = cosf(ang), sn = sinf(ang);
+                    v = cr < half ? qt[i] * cs - qt[half + i] * sn : qt[half + i] * cs + qt[i] * sn;
+                }
+            }
+        }
+        qs[r * qld + c] = v;
+    }
+    __syncthreads();
+    const long long tile = (long long)blockIdx.x * 4 + wave, j0 = lo + tile * 16;
+    const float *ring = step->state + ring_off;
+    const la_src k1 = {ring, (long long)(R + dr), 0, cap}, k2 = {ring + R, (long long)(R + dr), 0, cap};
+    long long rowpos[4];
+    float m[4], l[4];
+    la_f4 acc[NJ];
+#pragma unroll
+    for (int i = 0; i < 4; i++) { rowpos[i] = h0 + 4 * lq + i < H ? p : -1; m[i] = -INFINITY; l[i] = 0.f; }
+#pragma unroll
+    for (int j = 0; j < NJ; j++) acc[j] = la_f4{0.f, 0.f, 0.f, 0.f};
+    if (j0 <= p) la_tile<NJ>(qs, qld, pt, k1, k2, k1, R, dr, R, j0, p + 1, rowpos, window, scale, m, l, acc);
+    // partial of (tile, head): [m, l, o[R]]
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int h = h0 + 4 * lq + i;
+        if (h >= H) continue;
+        float *pp = part + ((long long)tile * H + h) * (R + 2);
+        if (lr == 0) { pp[0] = m[i]; pp[1] = l[i]; }
+#pragma unroll
+        for (int J = 0; J < NJ / 4; J++)
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++) {
+                const int c = 64 * J + 4 * lr + jj;
+                if (c < R) pp[2 + c] = acc[4 * J + jj][i];
+            }
+    }
+}
+// ol[h][c] = sum_tiles exp(m_t - M) o_t[c] / sum_tiles exp(m_t - M) l_t
+__global__ __launch_bounds__(256) void latent_combine_kernel(const ps_seq_step *step, const float *part, int H, int R, int window, int max_tiles, float *ol) {
+    const int h = blockIdx.x;
+    const long long p = step->pos0, lo = p - window + 1 > 0 ? p - window + 1 : 0;
+    int nt = (int)((p - lo) / 16 + 1);
+    if (nt > max_tiles) nt = max_tiles;
+    float M = -INFINITY;
+    for (int t = 0; t < nt; t++) M = fmaxf(M, part[((long long)t * H + h) * (R + 2)]);
+    float L = 0.f;
+    for (int t = 0; t < nt; t++) {
+        const float *pp = part + ((long long)t * H + h) * (R + 2);
+        L += pp[0] == -INFINITY ? 0.f : expf(pp[0] - M) * pp[1];
+    }
+    for (int c = threadIdx.x; c < R; c += 256) {
+        float a = 0.f;
+        for (int t = 0; t < nt; t++) {
+            const float *pp = part + ((long long)t * H + h) * (R + 2);
+            if (pp[0] != -INFINITY) a = fmaf(expf(pp[0] - M), pp[2 + c], a);
+        }
+        ol[(long long)h * R + c] = a / L;
+    }
+}
+
+bool psk_latent_absorbed_ok(int d, int dr, int dv, int R) { return R % 16 == 0 && dr % 16 == 0 && R <= 512 && (size_t)(16 * (R + dr + 4) + 4 * 16 * 17) * 4 <= 160 * 1024; }
+size_t psk_latent_absorbed_scratch(int H, int R, int window) { return ((size_t)((window + 15) / 16 + 4) * H * (R + 2) + (size_t)2 * H * R) * 4; }
+// q [H][d + dr] (row stride qstride) -> o [H * dv]; ukv: rows uk | uv of the expansion matrix [H d + H dv][R]; scratch from psk_latent_absorbed_scratch
+void psk_latent_absorbed(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, const float *q, int qstride, const ps_dense *ukv, const float *freq,
+                         int H, int d, int dr, int rot_dims, int dv, int R, int window, float scale, float *scratch, float *o) {
+    const int max_tiles = (window + 15) / 16 + 1; // (a window that does not start on a tile's edge touches one tile more)
+    float *qa = scratch, *ol = qa + (size_t)H * R, *part = ol + (size_t)H * R;
+    const bool bf = ukv->dtype == PS_BF16;
+    if (bf) hipLaunchKernelGGL(latent_fold_q_kernel<unsigned short>, dim3(H), dim3(256), 0, st, q, qstride, (const unsigned short *)ukv->data, d, R, qa);
+    else hipLaunchKernelGGL(latent_fold_q_kernel<float>, dim3(H), dim3(256), 0, st, q, qstride, (const float *)ukv->data, d, R, qa);
+    const size_t lds = (size_t)(16 * (R + dr + 4) + 4 * 16 * 17) * 4;
+    const dim3 grid((max_tiles + 3) / 4, (H + 15) / 16);
+    if (R <= 128) {
+        static unsigned long long mask = 0;
+        if (ps_first_on_device(&mask)) (void)hipFuncSetAttribute((const void *)latent_absorbed_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipLaunchKernelGGL(latent_absorbed_kernel<8>, grid, dim3(256), lds, st, step, (long long)ring_off, cap, qa, q, qstride, d, dr, rot_dims, freq, H, R, window, scale, part);
+    } else {
+        static unsigned long long mask = 0;
+        if (ps_first_on_device(&mask)) (void)hipFuncSetAttribute((const void *)latent_absorbed_kernel<32>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipLaunchKernelGGL(latent_absorbed_kernel<32>, grid, dim3(256), lds, st, step, (long long)ring_off, cap, qa, q, qstride, d, dr, rot_dims, freq, H, R, window, scale, part);
+    }
+    hipLaunchKernelGGL(latent_combine_kernel, dim3(H), dim3(256), 0, st, step, part, H, R, window, (int)grid.x * 4, ol);
+    const int rows = H * dv;
+    if (bf) hipLaunchKernelGGL(latent_unfold_v_kernel<unsigned short>, dim3((rows + 3) / 4), dim3(256), 0, st, ol, (const unsigned short *)ukv->data + (size_t)H * d * R, dv, R, rows, o);
+    else hipLaunchKernelGGL(latent_unfold_v_kernel<float>, dim3((rows + 3) / 4), dim3(256), 0, st, ol, (const float *)ukv->data + (size_t)H * d * R, dv, R, rows, o);
+}

@@ -39,7 +39,9 @@ struct psk_dense_args {
     int act = PSD_ACT_NONE;
     float act_p = 0.f, act_q = 0.f, alpha = 1.f; // xIELU: act_p = softplus(p), act_q = 1/2 + softplus(q)
     const float *mu = nullptr, *shift0 = nullptr;
-    int force_tiled = 0; // 1: the tiled mat-mul also for a few rows (A/B against the mat-vec)
+    int force_tiled = 0; // 1: the plain tiled mat-mul whatever the shape (A/B against the mat-vec and the wide mat-mul)
+    void *pack = nullptr; // scratch for the wide mat-mul's bfloat16 copy of A (T rounded up to 128 rows of K); without it the plain tiled kernel runs
+    size_t pack_bytes = 0;
 };
 int psk_dense(hipStream_t st, const psk_dense_args &a);
 void psk_dense_widen(hipStream_t st, const uint16_t *bf16, int64_t n, float *out);
@@ -83,3 +85,13 @@ void psk_latent_prep(hipStream_t st, const ps_seq_step *step, int64_t ring_off, 
 // first .. first + Nw - 1 where first = max(0, pos0 - window + 1) (the caller expands exactly these ring rows), rotated key parts from the ring.
 void psk_latent_attn(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, const float *q, int64_t ldq, const float *kv, int64_t ldkv,
                      const float *freq, int H, int d, int dr, int rot_dims, int dv, int kv_rank, int window, float scale, int T, float *o, int64_t ldo);
+// The same attention on the matrix cores (fp32 MFMA), 16 tokens of a head per wave; _ok: the sizes it takes (d, dr multiples of 16, dv of 4, dv <= 128).
+bool psk_latent_attn_mfma_ok(int d, int dr, int dv);
+void psk_latent_attn_mfma(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, const float *q, int64_t ldq, const float *kv, int64_t ldkv,
+                          const float *freq, int H, int d, int dr, int rot_dims, int dv, int kv_rank, int window, float scale, int T, float *o, int64_t ldo);
+// Single-token step in the absorbed form: nothing is expanded per key, the ring's latents are keys and values for all heads at once.
+// q [H][d + dr] (row stride qstride, rotated part not yet rotated) -> o [H * dv].  ukv: rows uk | uv.  _ok: kv_rank, dr multiples of 16, kv_rank <= 512.
+bool psk_latent_absorbed_ok(int d, int dr, int dv, int R);
+size_t psk_latent_absorbed_scratch(int H, int R, int window);
+void psk_latent_absorbed(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, const float *q, int qstride, const ps_dense *ukv, const float *freq,
+                         int H, int d, int dr, int rot_dims, int dv, int R, int window, float scale, float *scratch, float *o);

@@ -35,6 +35,9 @@ struct ps_hip_seq {
     float *x = nullptr, *hn = nullptr, *h = nullptr, *y = nullptr, *t1 = nullptr, *t2 = nullptr, *t3 = nullptr, *t4 = nullptr, *kvx = nullptr, *xn = nullptr,
           *logits = nullptr;
     int32_t *tokens = nullptr, *want = nullptr, *amax = nullptr, *ids = nullptr;
+    float *abs_scratch = nullptr; // the absorbed single-token attention's folded queries, attended latents and per-tile partials
+    void *pack = nullptr; // the wide mat-mul's bfloat16 operand copy
+    size_t pack_bytes = 0;
     int ids_cap = 0;
     int64_t n_t2q = 0; // t2: [max_batch][q_rank max] then the queries
     float *dbg_layers = nullptr;
@@ -141,7 +144,7 @@ int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) 
     n2 = std::max(n2, m->n_t2q + nq);
     m->zero_floats = off;
     for (auto &P : m->L)
-        if (P.d.kind == PS_MIX_LATENT) { P.off_ring = off; off += (int64_t)P.cap * (P.d.kv_rank + P.d.rot_dim); }
+        if (P.d.kind == PS_MIX_LATENT) { off = (off + 3) / 4 * 4; P.off_ring = off; off += (int64_t)P.cap * (P.d.kv_rank + P.d.rot_dim); } // (16-byte rows for the matrix-core kernels)
     m->state_floats = off;
     auto alloc = [&](void **p, size_t bytes) {
         if (ps_dev_malloc(p, bytes + 256) != hipSuccess) return false;
@@ -162,6 +165,23 @@ int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) 
          alloc((void **)&m->t3, B * std::max<int64_t>(n3, 1) * 4) && alloc((void **)&m->t4, B * std::max<int64_t>(n4, 1) * 4) &&
          alloc((void **)&m->kvx, std::max<int64_t>(nkv, 1) * 4) && alloc((void **)&m->xn, B * W * 4) && alloc((void **)&m->logits, B * (int64_t)desc->vocab * 4) &&
          alloc((void **)&m->tokens, B * 4) && alloc((void **)&m->want, B * 4) && alloc((void **)&m->amax, B * 4);
+    {
+        size_t ab = 0;
+        for (auto &P : m->L)
+            if (P.d.kind == PS_MIX_LATENT && psk_latent_absorbed_ok(P.d.dim, P.d.rot_dim, P.d.vdim, P.d.kv_rank))
+                ab = std::max(ab, psk_latent_absorbed_scratch(P.d.heads, P.d.kv_rank, P.d.window));
+        if (ab) ok = ok && alloc((void **)&m->abs_scratch, ab);
+    }
+    if (desc->compute == 0) { // the wide mat-mul's operand copy: the widest input of any matrix x a portion's rows, or the window's rows x the latent
+        int64_t kmax = W, kvrows = 0, kvk = 0;
+        for (auto &P : m->L) {
+            kmax = std::max<int64_t>({kmax, P.d.ff, P.d.heads * (int64_t)std::max(P.d.dim, P.d.vdim), P.d.q_rank, P.d.decay_rank});
+            if (P.d.kind == PS_MIX_LATENT) { kvrows = std::max<int64_t>(kvrows, P.d.window - 1 + B); kvk = std::max<int64_t>(kvk, P.d.kv_rank); }
+        }
+        const int64_t r128 = (B + 127) / 128 * 128, kv128 = (kvrows + 127) / 128 * 128;
+        m->pack_bytes = (size_t)std::max(r128 * kmax, kv128 * kvk) * 2;
+        ok = ok && alloc(&m->pack, m->pack_bytes);
+    }
     m->slot_state.assign(desc->n_slots, nullptr);
     m->slot_pos.assign(desc->n_slots, -1);
     for (int s = 0; ok && s < desc->n_slots; s++) ok = alloc((void **)&m->slot_state[s], (size_t)m->state_floats * 4);
@@ -217,7 +237,7 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
     psk_embed(st, D.embed, from_step ? nullptr : m->tokens, m->step, T, m->x, W);
     auto mm = [&](const ps_dense *w, const float *a, int64_t lda, float *out, int64_t ldo) {
         psk_dense_args g;
-        g.w = w; g.a = a; g.lda = lda; g.T = T; g.out = out; g.ldo = ldo; g.force_tiled = tiled;
+        g.w = w; g.a = a; g.lda = lda; g.T = T; g.out = out; g.ldo = ldo; g.force_tiled = tiled; g.pack = m->pack; g.pack_bytes = m->pack_bytes;
         return g;
     };
     for (int li = 0; li < D.n_layers; li++) {
@@ -260,14 +280,23 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
             psk_dense(st, mm(l.in_cat, m->h, W, m->t1, P.ncat));
             psk_latent_prep(st, m->step, P.off_ring, P.cap, m->t1, P.ncat, l.qnorm, l.kvnorm, D.norm_eps, l.q_rank, l.kv_rank, (int)dr, l.rot_dims, P.freq, T, cq, l.q_rank);
             psk_dense(st, mm(l.uq, cq, l.q_rank, q, nq));
-            { // the window's keys and values, expanded from the ring rows  max(0, pos0 - window + 1) .. pos0 + T - 1
+            const bool plain = (m->mode & 2) != 0, rows4 = (l.kv_rank + dr) % 4 == 0 && l.kv_rank % 4 == 0;
+            if (T == 1 && !plain && m->abs_scratch && psk_latent_absorbed_ok((int)d, (int)dr, (int)dv, l.kv_rank)) {
+                psk_latent_absorbed(st, m->step, P.off_ring, P.cap, q, (int)(d + dr), l.ukv, P.freq, (int)H, (int)d, (int)dr, l.rot_dims, (int)dv, l.kv_rank, l.window,
+                                    l.scale, m->abs_scratch, m->t3);
+            } else {
+                // the window's keys and values, expanded from the ring rows  max(0, pos0 - window + 1) .. pos0 + T - 1
                 auto g = mm(l.ukv, state + P.off_ring, rs, m->kvx, H * d + Hv);
                 g.a_step = m->step; g.a_row0 = -(int64_t)(l.window - 1); g.a_mod = P.cap;
                 g.T = any_pos ? l.window - 1 + T : (int)(std::min<int64_t>(pos0, l.window - 1) + T);
-                g.force_tiled = 1;
                 psk_dense(st, g);
+                if (!plain && rows4 && psk_latent_attn_mfma_ok((int)d, (int)dr, (int)dv))
+                    psk_latent_attn_mfma(st, m->step, P.off_ring, P.cap, q, nq, m->kvx, H * d + Hv, P.freq, (int)H, (int)d, (int)dr, l.rot_dims, (int)dv, l.kv_rank, l.window,
+                                         l.scale, T, m->t3, Hv);
+                else
+                    psk_latent_attn(st, m->step, P.off_ring, P.cap, q, nq, m->kvx, H * d + Hv, P.freq, (int)H, (int)d, (int)dr, l.rot_dims, (int)dv, l.kv_rank, l.window,
+                                    l.scale, T, m->t3, Hv);
             }
-            psk_latent_attn(st, m->step, P.off_ring, P.cap, q, nq, m->kvx, H * d + Hv, P.freq, (int)H, (int)d, (int)dr, l.rot_dims, (int)dv, l.kv_rank, l.window, l.scale, T, m->t3, Hv);
             psk_dense(st, mm(l.out, m->t3, Hv, m->y, W));
         }
         psk_norm_residual(st, m->x, m->y, l.norm1b, D.norm_offset, D.norm_eps, W, T);
@@ -290,7 +319,7 @@ static void seq_head(ps_hip_seq *m, const int32_t *idx, int rows) {
     const ps_seq_desc &D = m->d;
     psk_rmsnorm(st, m->x, D.width, idx, D.final_norm, D.norm_offset, D.norm_eps, D.width, rows, m->xn, D.width);
     psk_dense_args g;
-    g.w = D.head; g.a = m->xn; g.lda = D.width; g.T = rows; g.out = m->logits; g.ldo = D.vocab; g.alpha = D.logit_scale; g.force_tiled = (m->mode & 2) != 0;
+    g.w = D.head; g.a = m->xn; g.lda = D.width; g.T = rows; g.out = m->logits; g.ldo = D.vocab; g.alpha = D.logit_scale; g.force_tiled = (m->mode & 2) != 0; g.pack = m->pack; g.pack_bytes = m->pack_bytes;
     psk_dense(st, g);
     psk_argmax_rows(st, m->logits, D.vocab, rows, m->amax);
 }
@@ -377,8 +406,37 @@ int ps_hip_seq_decode_greedy(ps_hip_seq *m, int slot, int32_t token, int steps, 
 }
 
 int ps_hip_seq_bench_kernel(ps_hip_seq *m, int which, int T, int reps, double *us, double *bytes, double *flops) {
-    (void)m; (void)which; (void)T; (void)reps; (void)us; (void)bytes; (void)flops;
-    return seq_fail(m->ctx, "seq_bench_kernel: not built yet");
+    ps_hip_ctx *c = m->ctx;
+    if (T <= 0 || T > m->d.max_batch || reps <= 0 || which < 0 || which > 1) return seq_fail(c, "seq_bench_kernel: bad argument");
+    PS_CHECK(c, hipSetDevice(c->device));
+    std::vector<psk_dense_args> launches; // one per layer that has the matrix: every launch streams its own (cold) weights, as in a step
+    for (const LayerPlan &P : m->L) {
+        if (P.d.ff_kind != PS_FF_DENSE_XIELU) continue;
+        psk_dense_args g;
+        g.T = T; g.pack = m->pack; g.pack_bytes = m->pack_bytes;
+        if (which == 0) { g.w = P.d.ff_up; g.a = m->h; g.lda = m->d.width; g.out = m->t4; g.ldo = P.d.ff; g.act = PSD_ACT_XIELU; g.act_p = P.act_p; g.act_q = P.act_q; }
+        else { g.w = P.d.ff_down; g.a = m->t4; g.lda = P.d.ff; g.out = m->y; g.ldo = m->d.width; }
+        launches.push_back(g);
+    }
+    if (launches.empty()) return seq_fail(c, "seq_bench_kernel: no layer has a feed-forward");
+    psk_fill(c->stream, m->h, 0.01f, (int64_t)m->d.max_batch * m->d.width);
+    hipEvent_t e0, e1;
+    PS_CHECK(c, hipEventCreate(&e0));
+    PS_CHECK(c, hipEventCreate(&e1));
+    for (auto &g : launches) psk_dense(c->stream, g); // warm-up (code objects, attributes)
+    PS_CHECK(c, hipEventRecord(e0, c->stream));
+    for (int r = 0; r < reps; r++)
+        for (auto &g : launches) psk_dense(c->stream, g);
+    PS_CHECK(c, hipEventRecord(e1, c->stream));
+    PS_CHECK(c, hipEventSynchronize(e1));
+    float ms = 0.f;
+    PS_CHECK(c, hipEventElapsedTime(&ms, e0, e1));
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    *us = 1e3 * ms / ((double)reps * launches.size());
+    *bytes = (double)dense_bytes(launches[0].w);
+    *flops = 2.0 * T * (double)launches[0].w->N * (double)launches[0].w->K;
+    return 0;
 }
 
 } // extern "C"

@@ -29,7 +29,9 @@ CONFIGS = {
     "latent": synth.seq_config(40, 32, [L("latent_attention", None, heads=2, dim=12, vdim=20, q_rank=16, kv_rank=24, mask={"size": 6}, scale=0.4, **LAT)], taps=3),
     "ff": synth.seq_config(40, 32, [L("wkv", 24, heads=1, dim=8)], taps=2),
 }
-TOL = {"float32": 2e-4, "bfloat16": 6e-2}
+# float32: a few ulps of fp32 sums.  bfloat16: the operands of every matrix product are rounded to 8 bits of mantissa, which in models this
+# narrow (48 to 128 channels) leaves 1-3 % on a typical row and up to 7 % on the worst of a hundred rows, whatever the schedule
+TOL = {"float32": 2e-4, "bfloat16": 1e-1}
 
 
 def err(got, want):
@@ -172,7 +174,7 @@ def test_interleaved_requests_and_reused_slots(made):
         m.release(s)
 
 
-def peaked_latent_model(window, seed=0, second_layer=True):
+def peaked_latent_model(window, seed=0, second_layer=True, aligned=False):
     """A latent-attention model whose scores are made by hand: every token's embedding is a constant half (ones) and a token-specific half of
     +-1 (so the norm in front of the mixer changes nothing); queries and the shared rotated key part read the constant half only, so the rotated
     part of the score depends on the DISTANCE alone, 8 (cos(d) + cos(2 pi d / (window - 1))) for window - 1 = 44 k: largest for the token
@@ -180,6 +182,8 @@ def peaked_latent_model(window, seed=0, second_layer=True):
     token-specific half.  A key lost or gained at the edge therefore moves the output by a large fraction of itself."""
     rng = np.random.default_rng(seed)
     W, half, V, H, d, dv, qr, kr, dr = 16, 8, 32, 2, 4, 6, 4, 6, 4
+    if aligned:  # sizes the matrix-core attention kernels take (the prompt's and the absorbed single-token form); 4 of 16 rotated numbers turn
+        d, dv, kr, dr = 16, 8, 16, 16
     f1 = 2 * np.pi / (window - 1)
     mixer = dict(heads=H, dim=d, vdim=dv, q_rank=qr, kv_rank=kr, rot_dim=dr, rot={"base": float(1.0 / f1 ** 2), "dims": 4}, mask={"size": int(window)}, scale=2.0)
     layers = [synth.seq_layer("latent_attention", None, **mixer)] + ([synth.seq_layer("wkv", 24, heads=2, dim=8)] if second_layer else [])
@@ -194,7 +198,7 @@ def peaked_latent_model(window, seed=0, second_layer=True):
     c0 = dq[:, :half].sum(1).astype(np.float64)
     c0 = c0 / np.sqrt(np.mean(c0 * c0) + cfg["norm"]["eps"])       # the query latent of every token
     uq = rng.standard_normal((H, d + dr, qr)) * 0.1
-    uq[:, d:, :] = np.outer([2.0, 2.0, 0.0, 0.0], c0 / (c0 @ c0))   # rotated query part (2, 2, 0, 0) before the rotation
+    uq[:, d:, :] = np.outer([2.0, 2.0] + [0.0] * (dr - 2), c0 / (c0 @ c0))   # rotated query part (2, 2, 0, ...) before the rotation
     t["l0.mix.uq"] = uq.reshape(H * (d + dr), qr).astype(np.float32)
     dkv = np.zeros((kr + dr, W), np.float32)
     dkv[:kr, half:] = rng.standard_normal((kr, W - half)) * 0.5     # the latent reads the token-specific half
@@ -208,14 +212,15 @@ def _rows(got, want, lo):
     return [err(got[i:i + 1], want[i:i + 1]) for i in range(lo, len(want))]
 
 
+@pytest.mark.parametrize("aligned", [False, True])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_window_edges_in_prompts_and_in_decoding(made, dtype):
+def test_window_edges_in_prompts_and_in_decoding(made, dtype, aligned):
     """The plain statement with a window one shorter loses the edge key and is far off at every later position, one longer gains a key and is
     clearly off; the library agrees with the right one whether the edge passes over prompt tokens, portions' borders or decoded tokens, also
     when the ring of latents (window - 1 + 8 rows here) has wrapped."""
     window = 45
-    cfg, t = peaked_latent_model(window)
-    m, _, _ = made("peaked45", dtype, max_batch=8, cfg=cfg, tensors=t)
+    cfg, t = peaked_latent_model(window, aligned=aligned)
+    m, _, _ = made("peaked45%d" % aligned, dtype, max_batch=8, cfg=cfg, tensors=t)
     toks = tokens_for(cfg, 120, seed=3)
     want = seq_oracle.run(cfg, t, toks)
     assert np.median(_rows(seq_oracle.run(cfg, t, toks, window_override={0: window - 1}), want, window - 1)) > 0.3
@@ -225,12 +230,13 @@ def test_window_edges_in_prompts_and_in_decoding(made, dtype):
         assert max(_rows(got, want, 0)) < (1e-3 if dtype == "float32" else TOL[dtype]), sizes
 
 
-def test_far_key_among_hundreds_and_a_ring_that_wraps(made):
+@pytest.mark.parametrize("aligned", [False, True])
+def test_far_key_among_hundreds_and_a_ring_that_wraps(made, aligned):
     """window 309: the key 308 tokens back carries a large share of the weight.  A 330-token prompt in portions of 64, then 170 single tokens:
     the ring (372 rows) wraps, and the far key is first a prompt token, then a decoded one."""
     window = 309
-    cfg, t = peaked_latent_model(window, seed=1)
-    m, _, _ = made("peaked309", "float32", max_batch=64, cfg=cfg, tensors=t)
+    cfg, t = peaked_latent_model(window, seed=1, aligned=aligned)
+    m, _, _ = made("peaked309%d" % aligned, "float32", max_batch=64, cfg=cfg, tensors=t)
     toks = tokens_for(cfg, 500, seed=4)
     want = seq_oracle.run(cfg, t, toks)
     assert np.median(_rows(seq_oracle.run(cfg, t, toks, window_override={0: window - 1}), want, window - 1)) > 0.1
@@ -270,14 +276,20 @@ def test_greedy_generation_through_the_entry_point(made, dtype):
     sm.close()
 
 
-def test_tiled_matmul_and_matvec_agree(made):
-    m, cfg, t = made("aligned", "bfloat16", max_batch=16)
-    toks = tokens_for(cfg, 30, seed=8)
-    a = run_portions(m, toks, [1])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_matrix_core_forms_agree_with_the_plain_kernels(made, dtype):
+    """mode bit 1 keeps the per-key attention, the expanded single-token step and the 64 x 64 mat-mul: the wide mat-mul, the matrix-core
+    attention of a portion and the absorbed single-token attention must give the same logits (fp32: up to the order of sums)"""
+    m, cfg, t = made("aligned", dtype, max_batch=64)
+    toks = tokens_for(cfg, 150, seed=9)
+    fast = [run_portions(m, toks, sizes) for sizes in ([64], [1], [40, 1, 1, 1, 9])]
     m.set_mode(2)
-    b = run_portions(m, toks, [1])
+    plain = [run_portions(m, toks, sizes) for sizes in ([64], [1], [40, 1, 1, 1, 9])]
     m.set_mode(0)
-    assert err(a, b) < 1e-4  # same operand rounding, another order of the fp32 sums
+    want = seq_oracle.run(cfg, t, toks)
+    for a, b in zip(fast, plain):
+        assert err(a, b) < (1e-4 if dtype == "float32" else TOL[dtype])
+        assert err(a, want) < TOL[dtype]
 
 
 def test_refusals(ctx, tmp_path):
