@@ -153,15 +153,25 @@ static __device__ __forceinline__ void la_tile(const float *qs, int qld, float *
     const long long jk = j0 + lr < jend ? j0 + lr : jend - 1; // (a key row that exists; masked below)
     la_f4 s4 = {0.f, 0.f, 0.f, 0.f};
     const float *kr1 = la_row(k1, jk) + 4 * lq, *kr2 = la_row(k2, jk) + 4 * lq, *qr = qs + lr * qld + 4 * lq;
-    for (int g = 0; g < DK1; g += 16) {
-        const la_f4 b = *(const la_f4 *)(kr1 + g), a = *(const la_f4 *)(qr + g);
+    // eight 16-byte key pieces in flight per lane ahead of their 32 matrix instructions
+    for (int g0 = 0; g0 < DK1 + DK2; g0 += 128) {
+        la_f4 b[8], a[8];
 #pragma unroll
-        for (int e = 0; e < 4; e++) s4 = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], b[e], s4, 0, 0, 0);
-    }
-    for (int g = 0; g < DK2; g += 16) {
-        const la_f4 b = *(const la_f4 *)(kr2 + g), a = *(const la_f4 *)(qr + DK1 + g);
+        for (int u = 0; u < 8; u++) {
+            const int g = g0 + 16 * u;
+            b[u] = g < DK1 ? *(const la_f4 *)(kr1 + g) : (g < DK1 + DK2 ? *(const la_f4 *)(kr2 + (g - DK1)) : la_f4{0.f, 0.f, 0.f, 0.f});
+        }
 #pragma unroll
-        for (int e = 0; e < 4; e++) s4 = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], b[e], s4, 0, 0, 0);
+        for (int u = 0; u < 8; u++) {
+            const int g = g0 + 16 * u;
+            a[u] = g < DK1 + DK2 ? *(const la_f4 *)(qr + g) : la_f4{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            if (g0 + 16 * u < DK1 + DK2) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) s4 = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u][e], b[u][e], s4, 0, 0, 0);
+            }
     }
     const long long j = j0 + lr;
     float p[4], corr[4];
@@ -195,13 +205,20 @@ static __device__ __forceinline__ void la_tile(const float *qs, int qld, float *
         const long long jv = j0 + 4 * s + lq < jend ? j0 + 4 * s + lq : jend - 1; // (weight 0 beyond the end)
         vr[s] = la_row(vs, jv) + 4 * lr;
     }
+    la_f4 bn[4];
+#pragma unroll
+    for (int s = 0; s < 4; s++) bn[s] = 4 * lr < DV ? *(const la_f4 *)(vr[s]) : la_f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int J = 0; J < NJ / 4; J++) {
-        if (64 * J < DV) {
-            const bool in = 64 * J + 4 * lr < DV;
+        if (64 * J < DV) { // (uniform)
             la_f4 b[4];
 #pragma unroll
-            for (int s = 0; s < 4; s++) b[s] = in ? *(const la_f4 *)(vr[s] + 64 * J) : la_f4{0.f, 0.f, 0.f, 0.f};
+            for (int s = 0; s < 4; s++) b[s] = bn[s];
+            if (J + 1 < NJ / 4 && 64 * (J + 1) < DV) { // the next 64 columns' pieces are requested before this group's matrix instructions
+                const bool in = 64 * (J + 1) + 4 * lr < DV;
+#pragma unroll
+                for (int s = 0; s < 4; s++) bn[s] = in ? *(const la_f4 *)(vr[s] + 64 * (J + 1)) : la_f4{0.f, 0.f, 0.f, 0.f};
+            }
 #pragma unroll
             for (int jj = 0; jj < 4; jj++) {
                 la_f4 a = acc[4 * J + jj];
@@ -284,18 +301,22 @@ void psk_latent_attn_mfma(hipStream_t st, const ps_seq_step *step, int64_t ring_
 // qa[h][r] = sum_i q[h][i] Wuk[h * d + i][r]: a head's query folded into latent space.  One block per head, a thread per latent index.
 template <typename WT>
 __global__ __launch_bounds__(256) void latent_fold_q_kernel(const float *q, int qstride, const WT *wuk, int d, int R, float *qa) {
-    const int h = blockIdx.x;
+    __shared__ float part[4][64];
+    const int h = blockIdx.x, r = blockIdx.y * 64 + (threadIdx.x & 63), grp = threadIdx.x >> 6; // block: 64 latent indices x 4 slices of the head's rows
     const float *qh = q + (long long)h * qstride;
-    for (int r = threadIdx.x; r < R; r += 256) {
-        float a = 0.f;
-        for (int i = 0; i < d; i++) {
+    float a = 0.f;
+    if (r < R) {
+#pragma unroll 8
+        for (int i = grp; i < d; i += 4) {
             float w;
             if constexpr (sizeof(WT) == 2) w = __uint_as_float((unsigned)wuk[((long long)h * d + i) * R + r] << 16);
             else w = wuk[((long long)h * d + i) * R + r];
             a = fmaf(qh[i], w, a);
         }
-        qa[(long long)h * R + r] = a;
     }
+    part[grp][threadIdx.x & 63] = a;
+    __syncthreads();
+    if (grp == 0 && r < R) qa[(long long)h * R + r] = part[0][threadIdx.x] + part[1][threadIdx.x] + part[2][threadIdx.x] + part[3][threadIdx.x];
 }
 // o[h][x] = sum_r Wuv[h * dv + x][r] ol[h][r]: the value expansion of the attended latent.  A wave per output row.
 template <typename WT>
@@ -374,23 +395,33 @@ __global__ __launch_bounds__(256) void latent_absorbed_kernel(const ps_seq_step 
 }
 // ol[h][c] = sum_tiles exp(m_t - M) o_t[c] / sum_tiles exp(m_t - M) l_t
 __global__ __launch_bounds__(256) void latent_combine_kernel(const ps_seq_step *step, const float *part, int H, int R, int window, int max_tiles, float *ol) {
-    const int h = blockIdx.x;
+    extern __shared__ float wts[]; // [max_tiles] weights exp(m_t - M), then their l-weighted sum in red
+    __shared__ float red[4];
+    const int h = blockIdx.x, tid = threadIdx.x;
     const long long p = step->pos0, lo = p - window + 1 > 0 ? p - window + 1 : 0;
     int nt = (int)((p - lo) / 16 + 1);
     if (nt > max_tiles) nt = max_tiles;
-    float M = -INFINITY;
-    for (int t = 0; t < nt; t++) M = fmaxf(M, part[((long long)t * H + h) * (R + 2)]);
-    float L = 0.f;
-    for (int t = 0; t < nt; t++) {
+    float mx = -INFINITY;
+    for (int t = tid; t < nt; t += 256) mx = fmaxf(mx, part[((long long)t * H + h) * (R + 2)]);
+    mx = la_wave_max(mx);
+    if ((tid & 63) == 0) red[tid >> 6] = mx;
+    __syncthreads();
+    const float M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    float ls = 0.f;
+    for (int t = tid; t < nt; t += 256) {
         const float *pp = part + ((long long)t * H + h) * (R + 2);
-        L += pp[0] == -INFINITY ? 0.f : expf(pp[0] - M) * pp[1];
+        const float w = pp[0] == -INFINITY ? 0.f : expf(pp[0] - M);
+        wts[t] = w;
+        ls = fmaf(w, pp[1], ls);
     }
-    for (int c = threadIdx.x; c < R; c += 256) {
+    ls = la_wave_sum(ls);
+    if ((tid & 63) == 0) red[tid >> 6] = ls;
+    __syncthreads();
+    const float L = red[0] + red[1] + red[2] + red[3];
+    for (int c = tid; c < R; c += 256) {
         float a = 0.f;
-        for (int t = 0; t < nt; t++) {
-            const float *pp = part + ((long long)t * H + h) * (R + 2);
-            if (pp[0] != -INFINITY) a = fmaf(expf(pp[0] - M), pp[2 + c], a);
-        }
+        for (int t = 0; t < nt; t++) a = fmaf(wts[t], part[((long long)t * H + h) * (R + 2) + 2 + c], a);
         ol[(long long)h * R + c] = a / L;
     }
 }
@@ -403,8 +434,8 @@ void psk_latent_absorbed(hipStream_t st, const ps_seq_step *step, int64_t ring_o
     const int max_tiles = (window + 15) / 16 + 1; // (a window that does not start on a tile's edge touches one tile more)
     float *qa = scratch, *ol = qa + (size_t)H * R, *part = ol + (size_t)H * R;
     const bool bf = ukv->dtype == PS_BF16;
-    if (bf) hipLaunchKernelGGL(latent_fold_q_kernel<unsigned short>, dim3(H), dim3(256), 0, st, q, qstride, (const unsigned short *)ukv->data, d, R, qa);
-    else hipLaunchKernelGGL(latent_fold_q_kernel<float>, dim3(H), dim3(256), 0, st, q, qstride, (const float *)ukv->data, d, R, qa);
+    if (bf) hipLaunchKernelGGL(latent_fold_q_kernel<unsigned short>, dim3(H, (R + 63) / 64), dim3(256), 0, st, q, qstride, (const unsigned short *)ukv->data, d, R, qa);
+    else hipLaunchKernelGGL(latent_fold_q_kernel<float>, dim3(H, (R + 63) / 64), dim3(256), 0, st, q, qstride, (const float *)ukv->data, d, R, qa);
     const size_t lds = (size_t)(16 * (R + dr + 4) + 4 * 16 * 17) * 4;
     const dim3 grid((max_tiles + 3) / 4, (H + 15) / 16);
     if (R <= 128) {
@@ -416,7 +447,7 @@ void psk_latent_absorbed(hipStream_t st, const ps_seq_step *step, int64_t ring_o
         if (ps_first_on_device(&mask)) (void)hipFuncSetAttribute((const void *)latent_absorbed_kernel<32>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         hipLaunchKernelGGL(latent_absorbed_kernel<32>, grid, dim3(256), lds, st, step, (long long)ring_off, cap, qa, q, qstride, d, dr, rot_dims, freq, H, R, window, scale, part);
     }
-    hipLaunchKernelGGL(latent_combine_kernel, dim3(H), dim3(256), 0, st, step, part, H, R, window, (int)grid.x * 4, ol);
+    hipLaunchKernelGGL(latent_combine_kernel, dim3(H), dim3(256), (size_t)grid.x * 4 * 4, st, step, part, H, R, window, (int)grid.x * 4, ol);
     const int rows = H * dv;
     if (bf) hipLaunchKernelGGL(latent_unfold_v_kernel<unsigned short>, dim3((rows + 3) / 4), dim3(256), 0, st, ol, (const unsigned short *)ukv->data + (size_t)H * d * R, dv, R, rows, o);
     else hipLaunchKernelGGL(latent_unfold_v_kernel<float>, dim3((rows + 3) / 4), dim3(256), 0, st, ol, (const float *)ukv->data + (size_t)H * d * R, dv, R, rows, o);

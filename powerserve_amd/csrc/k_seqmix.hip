@@ -111,15 +111,63 @@ void psk_copy(hipStream_t st, const float *src, float *dst, int64_t n) {
     hipLaunchKernelGGL(sq_copy_kernel, dim3((unsigned)min((long long)((n + 255) / 256), 4096ll)), dim3(256), 0, st, src, dst, (long long)n);
 }
 
+
+// A single token's sublayer boundary in one launch (one block):  x += y / rms(y) * (offset + wb)   (where y is given), then, where wn is given,
+// h = conv(x / rms(x) * (offset + wn)) with the convolution's residual form and its tail brought up to date -- three launches of the kernels above.
+__global__ __launch_bounds__(1024) void sq_boundary1_kernel(const ps_seq_step *step, float *x, const float *y, const float *wb, const float *wn, const float *cw,
+                                                            int taps, long long tail_off, float offset, float eps, long long n, float *h) {
+    __shared__ float red[16];
+    const int tid = threadIdx.x, nw = blockDim.x >> 6;
+    auto block_sum = [&](float v) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+        __syncthreads();
+        if ((tid & 63) == 0) red[tid >> 6] = v;
+        __syncthreads();
+        float s = 0.f;
+        for (int w = 0; w < nw; w++) s += red[w];
+        return s;
+    };
+    float s2 = 0.f;
+    if (y) {
+        float s1 = 0.f;
+        for (long long i = tid; i < n; i += blockDim.x) s1 += y[i] * y[i];
+        const float inv = 1.f / sqrtf(block_sum(s1) / (float)n + eps);
+        for (long long i = tid; i < n; i += blockDim.x) {
+            const float v = x[i] + y[i] * inv * (offset + wb[i]);
+            x[i] = v;
+            s2 += v * v;
+        }
+    } else {
+        for (long long i = tid; i < n; i += blockDim.x) s2 += x[i] * x[i];
+    }
+    if (!wn) return;
+    const float inv = 1.f / sqrtf(block_sum(s2) / (float)n + eps);
+    float *tail = step->state + tail_off;
+    for (long long c = tid; c < n; c += blockDim.x) { // (a thread re-reads only what it wrote itself)
+        const float v = x[c] * inv * (offset + wn[c]);
+        float s = cw[c * taps + taps - 1] * v;
+        for (int j = 0; j < taps - 1; j++) s = fmaf(cw[c * taps + j], tail[(long long)j * n + c], s);
+        h[c] = v + s;
+        for (int j = 0; j + 1 < taps - 1; j++) tail[(long long)j * n + c] = tail[(long long)(j + 1) * n + c];
+        if (taps > 1) tail[(long long)(taps - 2) * n + c] = v;
+    }
+}
+void psk_boundary1(hipStream_t st, const ps_seq_step *step, float *x, const float *y, const float *wb, const float *wn, const float *cw, int taps, int64_t tail_off,
+                   float offset, float eps, int64_t n, float *h) {
+    hipLaunchKernelGGL(sq_boundary1_kernel, dim3(1), dim3(n >= 2048 ? 1024 : 256), 0, st, step, x, y, wb, wn, cw, taps, (long long)tail_off, offset, eps, (long long)n, h);
+}
+
 // ---------------------------------------------------------------------------------------------------- recurrent scans
-#define SQ_NR 16 // state rows per lane
+typedef float sq_f4 __attribute__((ext_vector_type(4)));
+#define SQ_NR 16 // state rows per lane (lane s of a column holds rows 16 s .. 16 s + 15: its per-token vectors are four 16-byte LDS reads each)
 #define SQ_TC 8  // tokens staged per round
 static inline int sq_lanes_per_col(int d) { int R = 1; while (R * SQ_NR < d) R *= 2; return R; }
 
 // LDS: rs, ks, ws [TC][dp] (dp = NR * R, rows >= d zero), sc [TC] (sum_i r_i bonus_i k_i)
 __global__ __launch_bounds__(256) void sq_wkv_scan_kernel(const ps_seq_step *step, long long state_off, const float *r, const float *k, const float *v, const float *z,
                                                           long long ld, const float *bonus, int d, int R, int T, float *o, long long ldo) {
-    extern __shared__ float lds[];
+    extern __shared__ __attribute__((aligned(16))) float lds[];
     const int dp = SQ_NR * R, cpb = 256 / R;
     float *rs = lds, *ks = rs + SQ_TC * dp, *ws = ks + SQ_TC * dp, *sc = ws + SQ_TC * dp;
     const int h = blockIdx.y, tid = threadIdx.x, s = tid % R, j = blockIdx.x * cpb + tid / R;
@@ -128,7 +176,7 @@ __global__ __launch_bounds__(256) void sq_wkv_scan_kernel(const ps_seq_step *ste
     float S[SQ_NR];
 #pragma unroll
     for (int m = 0; m < SQ_NR; m++) {
-        const int i = s + R * m;
+        const int i = s * SQ_NR + m;
         S[m] = (col && i < d) ? S0[(long long)i * d + j] : 0.f;
     }
     const long long hb = (long long)h * d;
@@ -163,13 +211,16 @@ __global__ __launch_bounds__(256) void sq_wkv_scan_kernel(const ps_seq_step *ste
 #pragma unroll
         for (int t = 0; t < SQ_TC; t++) {
             if (t < nt) {
-                const float *rt = rs + t * dp, *kt = ks + t * dp, *wt = ws + t * dp;
+                const sq_f4 *rt = (const sq_f4 *)(rs + t * dp + s * SQ_NR), *kt = (const sq_f4 *)(ks + t * dp + s * SQ_NR), *wt = (const sq_f4 *)(ws + t * dp + s * SQ_NR);
                 float p = 0.f;
 #pragma unroll
-                for (int m = 0; m < SQ_NR; m++) {
-                    const int i = s + R * m;
-                    p = fmaf(rt[i], S[m], p);
-                    S[m] = fmaf(wt[i], S[m], kt[i] * vj[t]);
+                for (int m4 = 0; m4 < SQ_NR / 4; m4++) {
+                    const sq_f4 r4 = rt[m4], k4 = kt[m4], w4 = wt[m4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        p = fmaf(r4[e], S[4 * m4 + e], p);
+                        S[4 * m4 + e] = fmaf(w4[e], S[4 * m4 + e], k4[e] * vj[t]);
+                    }
                 }
                 for (int x = 1; x < R; x <<= 1) p += __shfl_xor(p, x, 64);
                 if (col && s == 0) o[(long long)(t0 + t) * ldo + hb + j] = fmaf(vj[t], sc[t], p);
@@ -178,7 +229,7 @@ __global__ __launch_bounds__(256) void sq_wkv_scan_kernel(const ps_seq_step *ste
     }
 #pragma unroll
     for (int m = 0; m < SQ_NR; m++) {
-        const int i = s + R * m;
+        const int i = s * SQ_NR + m;
         if (col && i < d) S0[(long long)i * d + j] = S[m];
     }
 }
@@ -194,7 +245,7 @@ void psk_wkv_scan(hipStream_t st, const ps_seq_step *step, int64_t state_off, co
 __global__ __launch_bounds__(256) void sq_delta_scan_kernel(const ps_seq_step *step, long long state_off, const float *q, const float *k, const float *v,
                                                             const float *braw, const float *araw, long long ld, long long ldb, const float *a_log, const float *dt_bias, int H,
                                                             int KH, int d, int dv, int R, int T, float *o, long long ldo) {
-    extern __shared__ float lds[];
+    extern __shared__ __attribute__((aligned(16))) float lds[];
     const int dp = SQ_NR * R, cpb = 256 / R;
     float *qs = lds, *ks = qs + SQ_TC * dp, *gs = ks + SQ_TC * dp, *bs = gs + SQ_TC, *kq = bs + SQ_TC;
     const int h = blockIdx.y, tid = threadIdx.x, s = tid % R, j = blockIdx.x * cpb + tid / R;
@@ -203,7 +254,7 @@ __global__ __launch_bounds__(256) void sq_delta_scan_kernel(const ps_seq_step *s
     float S[SQ_NR];
 #pragma unroll
     for (int m = 0; m < SQ_NR; m++) {
-        const int i = s + R * m;
+        const int i = s * SQ_NR + m;
         S[m] = (col && i < d) ? S0[(long long)i * dv + j] : 0.f;
     }
     const long long qb = (long long)(h / (H / KH)) * d, vb = (long long)h * dv;
@@ -253,15 +304,20 @@ __global__ __launch_bounds__(256) void sq_delta_scan_kernel(const ps_seq_step *s
 #pragma unroll
         for (int t = 0; t < SQ_TC; t++) {
             if (t < nt) {
-                const float *qt = qs + t * dp, *kt = ks + t * dp;
+                const sq_f4 *qt = (const sq_f4 *)(qs + t * dp + s * SQ_NR), *kt = (const sq_f4 *)(ks + t * dp + s * SQ_NR);
                 const float g = gs[t];
+                sq_f4 k4[SQ_NR / 4];
                 float p1 = 0.f, p2 = 0.f;
 #pragma unroll
-                for (int m = 0; m < SQ_NR; m++) {
-                    const int i = s + R * m;
-                    S[m] *= g;
-                    p1 = fmaf(kt[i], S[m], p1);
-                    p2 = fmaf(qt[i], S[m], p2);
+                for (int m4 = 0; m4 < SQ_NR / 4; m4++) {
+                    const sq_f4 q4 = qt[m4];
+                    k4[m4] = kt[m4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        S[4 * m4 + e] *= g;
+                        p1 = fmaf(k4[m4][e], S[4 * m4 + e], p1);
+                        p2 = fmaf(q4[e], S[4 * m4 + e], p2);
+                    }
                 }
                 for (int x = 1; x < R; x <<= 1) {
                     p1 += __shfl_xor(p1, x, 64);
@@ -269,14 +325,16 @@ __global__ __launch_bounds__(256) void sq_delta_scan_kernel(const ps_seq_step *s
                 }
                 const float u = bs[t] * (vj[t] - p1);
 #pragma unroll
-                for (int m = 0; m < SQ_NR; m++) S[m] = fmaf(kt[s + R * m], u, S[m]);
+                for (int m4 = 0; m4 < SQ_NR / 4; m4++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) S[4 * m4 + e] = fmaf(k4[m4][e], u, S[4 * m4 + e]);
                 if (col && s == 0) o[(long long)(t0 + t) * ldo + vb + j] = fmaf(u, kq[t], p2); // S_new^T q = (g S)^T q + u (k . q)
             }
         }
     }
 #pragma unroll
     for (int m = 0; m < SQ_NR; m++) {
-        const int i = s + R * m;
+        const int i = s * SQ_NR + m;
         if (col && i < d) S0[(long long)i * dv + j] = S[m];
     }
 }

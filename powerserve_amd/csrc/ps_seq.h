@@ -60,6 +60,9 @@ void psk_norm_residual(hipStream_t st, float *x, const float *y, const float *w,
 // (a residual around the convolution), mode 1: f = silu(sum).  The tail is brought up to date behind it.
 void psk_causal_conv(hipStream_t st, const ps_seq_step *step, int64_t tail_off, const float *in, int64_t ldi, const float *w, int taps, int mode,
                      int64_t C, int T, float *out, int64_t ldo);
+// One token's sublayer boundary fused: x += norm_b(y) (y may be NULL), then h = conv(norm(x)) in the residual form with the tail update (wn may be NULL: stop after x)
+void psk_boundary1(hipStream_t st, const ps_seq_step *step, float *x, const float *y, const float *wb, const float *wn, const float *cw, int taps, int64_t tail_off,
+                   float offset, float eps, int64_t n, float *h);
 // state row copy: (step->state + off)[0..n) = src[0..n)
 void psk_state_store(hipStream_t st, const ps_seq_step *step, int64_t off, const float *src, int64_t n);
 void psk_fill(hipStream_t st, float *p, float v, int64_t n);

@@ -240,12 +240,24 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
         g.w = w; g.a = a; g.lda = lda; g.T = T; g.out = out; g.ldo = ldo; g.force_tiled = tiled; g.pack = m->pack; g.pack_bytes = m->pack_bytes;
         return g;
     };
+    // a sublayer boundary: x += norm_b(y) (after a sublayer), then h = conv(norm(x)) (in front of the next one); one launch for a single token
+    auto boundary = [&](const float *y, const float *wb, const float *wn, const float *cw, int64_t tail_off) {
+        if (T == 1 && !tiled) {
+            psk_boundary1(st, m->step, m->x, y, wb, wn, cw, D.canon_taps, tail_off, D.norm_offset, D.norm_eps, W, m->h);
+            return;
+        }
+        if (y) psk_norm_residual(st, m->x, y, wb, D.norm_offset, D.norm_eps, W, T);
+        if (wn) {
+            psk_rmsnorm(st, m->x, W, nullptr, wn, D.norm_offset, D.norm_eps, W, T, m->hn, W);
+            psk_causal_conv(st, m->step, tail_off, m->hn, W, cw, D.canon_taps, 0, W, T, m->h, W);
+        }
+    };
+    boundary(nullptr, nullptr, m->L[0].d.norm1, m->L[0].d.canon1, m->L[0].off_canon1);
     for (int li = 0; li < D.n_layers; li++) {
         const LayerPlan &P = m->L[li];
         const ps_seq_layer &l = P.d;
         const int64_t H = l.heads, d = l.dim, dv = l.vdim;
-        psk_rmsnorm(st, m->x, W, nullptr, l.norm1, D.norm_offset, D.norm_eps, W, T, m->hn, W);
-        psk_causal_conv(st, m->step, P.off_canon1, m->hn, W, l.canon1, D.canon_taps, 0, W, T, m->h, W);
+        const LayerPlan *next = li + 1 < D.n_layers ? &m->L[li + 1] : nullptr;
         if (l.kind == PS_MIX_WKV) {
             const int64_t Hd = H * d, NW = 5 * Hd;
             const ps_dense *ws[4] = {l.in_r, l.in_k, l.in_v, l.in_g};
@@ -299,15 +311,17 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
             }
             psk_dense(st, mm(l.out, m->t3, Hv, m->y, W));
         }
-        psk_norm_residual(st, m->x, m->y, l.norm1b, D.norm_offset, D.norm_eps, W, T);
+        const float *nn = next ? next->d.norm1 : nullptr, *nc = next ? next->d.canon1 : nullptr;
+        const int64_t no = next ? next->off_canon1 : 0;
         if (l.ff_kind == PS_FF_DENSE_XIELU) {
-            psk_rmsnorm(st, m->x, W, nullptr, l.norm2, D.norm_offset, D.norm_eps, W, T, m->hn, W);
-            psk_causal_conv(st, m->step, P.off_canon2, m->hn, W, l.canon2, D.canon_taps, 0, W, T, m->h, W);
+            boundary(m->y, l.norm1b, l.norm2, l.canon2, P.off_canon2);
             auto g = mm(l.ff_up, m->h, W, m->t4, l.ff);
             g.act = PSD_ACT_XIELU; g.act_p = P.act_p; g.act_q = P.act_q;
             psk_dense(st, g);
             psk_dense(st, mm(l.ff_down, m->t4, l.ff, m->y, W));
-            psk_norm_residual(st, m->x, m->y, l.norm2b, D.norm_offset, D.norm_eps, W, T);
+            boundary(m->y, l.norm2b, nn, nc, no);
+        } else {
+            boundary(m->y, l.norm1b, nn, nc, no);
         }
         if (m->dbg_layers && !any_pos) psk_copy(st, m->x, m->dbg_layers + (int64_t)li * D.max_batch * W, (int64_t)T * W);
     }
