@@ -141,7 +141,7 @@ def build(force: bool = False, verbose: bool = True, contract: bool = True, time
     return so
 
 
-HOST_SOURCES = ["json_gguf.cpp", "graph.cpp", "hip_backend.cpp", "model.cpp", "speculative.cpp", "sampler.cpp"]
+HOST_SOURCES = ["json_gguf.cpp", "graph.cpp", "hip_backend.cpp", "model.cpp", "speculative.cpp", "sampler.cpp", "seq_model.cpp"]
 
 
 def build_host(force: bool = False, verbose: bool = True) -> str:

@@ -77,6 +77,10 @@ const JsonValue &JsonValue::at(const std::string &k) const {
     if (kind != OBJ || it == obj.end()) throw std::runtime_error("json: missing key '" + k + "'");
     return it->second;
 }
+JsonValue JsonValue::parse_text(const std::string &text) {
+    JP p{text};
+    return p.val();
+}
 JsonValue JsonValue::parse_file(const std::string &path) {
     std::ifstream f(path);
     if (!f.good()) throw std::runtime_error("cannot open " + path);

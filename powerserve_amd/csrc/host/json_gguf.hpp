@@ -20,6 +20,7 @@ struct JsonValue {
     const JsonValue &at(const std::string &k) const;
     bool contains(const std::string &k) const { return kind == OBJ && obj.count(k); }
     static JsonValue parse_file(const std::string &path);
+    static JsonValue parse_text(const std::string &text);
 };
 
 struct GGUFTensor {

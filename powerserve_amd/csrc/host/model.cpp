@@ -1,4 +1,6 @@
 #include "model.hpp"
+#include "seq_model.hpp"
+#include <filesystem>
 
 #include <cmath>
 #include <cstring>
@@ -326,6 +328,8 @@ auto Model::generate(const std::vector<Token> &prompt, int steps, size_t batch_s
 
 auto load_model(const std::string &model_dir, const std::shared_ptr<Platform> &platform, int device, size_t max_batch, int n_ctx_cap)
     -> std::shared_ptr<Model> {
+    if (is_seq_model_dir(model_dir) && !std::filesystem::exists(model_dir + "/model.json"))
+        POWERSERVE_ABORT(model_dir + " holds a layer-list model (config.json + model.safetensors): load it with load_seq_model");
     auto config = std::make_shared<ModelConfig>(model_dir + "/model.json");
     if (n_ctx_cap > 0) config->llm.seq_len = (uint32_t)n_ctx_cap; // explicit cap: the FP32 KV cache is sized by n_ctx
     if (config->arch != "llama" && config->arch != "qwen2") POWERSERVE_ABORT("unknown model type: " + config->arch);

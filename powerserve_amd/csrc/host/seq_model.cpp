@@ -1,0 +1,306 @@
+#include "seq_model.hpp"
+
+#include <cstring>
+#include <fcntl.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+namespace powerserve {
+
+// ---------------------------------------------------------------- safetensors
+SafeTensorsFile::SafeTensorsFile(const std::string &path) : m_path(path) {
+    int fd = open(path.c_str(), O_RDONLY);
+    if (fd < 0) POWERSERVE_ABORT("cannot open " + path);
+    struct stat st;
+    if (fstat(fd, &st) != 0 || st.st_size < 8) { close(fd); POWERSERVE_ABORT(path + ": not a safetensors file"); }
+    m_size = (size_t)st.st_size;
+    m_map = mmap(nullptr, m_size, PROT_READ, MAP_PRIVATE, fd, 0);
+    close(fd);
+    if (m_map == MAP_FAILED) { m_map = nullptr; POWERSERVE_ABORT("mmap failed: " + path); }
+    uint64_t n = 0;
+    memcpy(&n, m_map, 8);
+    if (n > m_size - 8) POWERSERVE_ABORT(path + ": header longer than the file");
+    try {
+        const JsonValue j = JsonValue::parse_text(std::string((const char *)m_map + 8, (size_t)n));
+        const char *base = (const char *)m_map + 8 + n;
+        const size_t room = m_size - 8 - (size_t)n;
+        for (const auto &[name, v] : j.obj) {
+            if (name == "__metadata__") continue;
+            SafeTensor t;
+            t.dtype = v.at("dtype").str;
+            for (const auto &s : v.at("shape").arr) t.shape.push_back((int64_t)s.num);
+            const auto &off = v.at("data_offsets").arr;
+            const size_t a = (size_t)off.at(0).num, b = (size_t)off.at(1).num;
+            const size_t es = t.dtype == "BF16" || t.dtype == "F16" ? 2 : (t.dtype == "F32" || t.dtype == "I32" ? 4 : 0);
+            if (!es) throw std::runtime_error("tensor " + name + ": unsupported dtype " + t.dtype);
+            if (b < a || b > room || b - a != (size_t)t.numel() * es) throw std::runtime_error("tensor " + name + ": data_offsets do not fit its shape");
+            t.data = base + a;
+            t.nbytes = b - a;
+            tensors[name] = t;
+        }
+    } catch (const std::exception &e) { POWERSERVE_ABORT(path + ": " + e.what()); }
+}
+SafeTensorsFile::~SafeTensorsFile() { if (m_map) munmap(m_map, m_size); }
+const SafeTensor &SafeTensorsFile::at(const std::string &name) const {
+    auto it = tensors.find(name);
+    if (it == tensors.end()) POWERSERVE_ABORT(m_path + ": tensor " + name + " is missing");
+    return it->second;
+}
+std::vector<float> SafeTensorsFile::f32(const std::string &name) const {
+    const SafeTensor &t = at(name);
+    std::vector<float> out((size_t)t.numel());
+    if (t.dtype == "F32") memcpy(out.data(), t.data, t.nbytes);
+    else if (t.dtype == "BF16") {
+        const uint16_t *b = (const uint16_t *)t.data;
+        for (size_t i = 0; i < out.size(); i++) { const uint32_t u = (uint32_t)b[i] << 16; memcpy(&out[i], &u, 4); }
+    } else POWERSERVE_ABORT("tensor " + name + ": " + t.dtype + " where a float tensor is expected");
+    return out;
+}
+std::vector<uint16_t> SafeTensorsFile::bf16_bits(const std::string &name) const {
+    const SafeTensor &t = at(name);
+    if (t.dtype != "BF16") POWERSERVE_ABORT("tensor " + name + " is " + t.dtype + ": the dense path takes bfloat16 matrices");
+    const uint16_t *b = (const uint16_t *)t.data;
+    return std::vector<uint16_t>(b, b + t.numel());
+}
+
+// ---------------------------------------------------------------- device copies
+static void hip_ok(ps_hip_ctx *c, int rc, const char *what) {
+    if (rc != 0) POWERSERVE_ABORT(std::string(what) + ": " + ps_hip_last_error(c));
+}
+const float *SeqUploader::vec(const std::vector<float> &a) {
+    void *p = nullptr;
+    hip_ok(ctx, ps_hip_malloc(ctx, std::max<size_t>(a.size(), 4) * 4, &p), "ps_hip_malloc");
+    vecs.push_back(p);
+    hip_ok(ctx, ps_hip_memcpy_h2d(ctx, p, a.data(), a.size() * 4), "ps_hip_memcpy_h2d");
+    return (const float *)p;
+}
+const ps_dense *SeqUploader::mat(const std::vector<uint16_t> &bits, int64_t rows, int64_t cols) {
+    POWERSERVE_ASSERT((int64_t)bits.size() == rows * cols);
+    ps_dense *w = nullptr;
+    hip_ok(ctx, ps_hip_dense_upload(ctx, bits.data(), rows, cols, as_f32 ? 1 : 0, &w), "ps_hip_dense_upload");
+    mats.push_back(w);
+    return w;
+}
+void SeqUploader::free_all() {
+    for (auto *w : mats) ps_hip_dense_free(ctx, w);
+    for (auto *p : vecs) ps_hip_free(ctx, p);
+    mats.clear();
+    vecs.clear();
+}
+
+// ---------------------------------------------------------------- Ranutar: configuration + tensors -> layer descriptors
+namespace {
+int64_t rows_of(const SafeTensorsFile &st, const std::string &n) { return st.at(n).shape.at(0); }
+int64_t cols_of(const SafeTensorsFile &st, const std::string &n) { return st.at(n).shape.at(1); }
+const ps_dense *mat1(const SafeTensorsFile &st, SeqUploader &up, const std::string &n) { return up.mat(st.bf16_bits(n), rows_of(st, n), cols_of(st, n)); }
+const ps_dense *mat_rows(const SafeTensorsFile &st, SeqUploader &up, const std::vector<std::string> &names) { // the matrices stacked by rows
+    std::vector<uint16_t> all;
+    int64_t rows = 0;
+    const int64_t cols = cols_of(st, names[0]);
+    for (const auto &n : names) {
+        if (cols_of(st, n) != cols) POWERSERVE_ABORT("tensor " + n + ": input size differs from " + names[0]);
+        auto b = st.bf16_bits(n);
+        all.insert(all.end(), b.begin(), b.end());
+        rows += rows_of(st, n);
+    }
+    return up.mat(all, rows, cols);
+}
+std::vector<float> expect(const SafeTensorsFile &st, const std::string &n, int64_t r, int64_t c) {
+    const auto &t = st.at(n);
+    if (t.shape.size() != 2 || t.shape[0] != r || t.shape[1] != c) POWERSERVE_ABORT("tensor " + n + ": its shape is not what the configuration gives");
+    return st.f32(n);
+}
+
+void ranutar(const JsonValue &cfg, const SafeTensorsFile &st, SeqUploader &up, std::vector<ps_seq_layer> &layers, ps_seq_desc &d) {
+    d.width = (int32_t)cfg.at("width").num;
+    d.vocab = (int32_t)cfg.at("vocab").num;
+    d.canon_taps = (int32_t)cfg.at("canon").at("taps").num;
+    d.norm_eps = (float)cfg.at("norm").at("eps").num;
+    d.norm_offset = 1.0f;
+    d.logit_scale = (float)cfg.at("logit_scale").num;
+    d.embed = mat1(st, up, "embed");
+    d.head = mat1(st, up, "head");
+    d.final_norm = up.vec(st.f32("final.norm"));
+    const auto &ls = cfg.at("layers").arr;
+    for (size_t i = 0; i < ls.size(); i++) {
+        const JsonValue &lc = ls[i], &mc = lc.at("mixer");
+        const std::string p = "l" + std::to_string(i) + ".", m = p + "mix.", kind = lc.at("type").str;
+        ps_seq_layer L{};
+        L.norm1 = up.vec(st.f32(p + "norm1"));
+        L.norm1b = up.vec(st.f32(p + "norm1b"));
+        L.canon1 = up.vec(expect(st, p + "canon1", d.width, d.canon_taps));
+        if (lc.contains("mlp") && lc.at("mlp").kind == JsonValue::OBJ) {
+            const JsonValue &f = lc.at("mlp");
+            if (f.at("kind").str != "dense") POWERSERVE_ABORT("layer " + std::to_string(i) + ": feed-forward kind " + f.at("kind").str + " is not known");
+            L.ff_kind = PS_FF_DENSE_XIELU;
+            L.ff = (int32_t)f.at("ff").num;
+            L.norm2 = up.vec(st.f32(p + "norm2"));
+            L.norm2b = up.vec(st.f32(p + "norm2b"));
+            L.canon2 = up.vec(expect(st, p + "canon2", d.width, d.canon_taps));
+            const auto act = st.f32(p + "mlp.act");
+            L.ff_act_p = act.at(0);
+            L.ff_act_q = act.at(1);
+            L.ff_up = mat1(st, up, p + "mlp.up");
+            L.ff_down = mat1(st, up, p + "mlp.down");
+        }
+        L.heads = (int32_t)mc.at("heads").num;
+        L.dim = (int32_t)mc.at("dim").num;
+        if (kind == "wkv") {
+            L.kind = PS_MIX_WKV;
+            L.vdim = L.dim;
+            L.decay_rank = (int32_t)rows_of(st, m + "w1");
+            L.in_r = mat1(st, up, m + "r"); L.in_k = mat1(st, up, m + "k"); L.in_v = mat1(st, up, m + "v"); L.in_g = mat1(st, up, m + "g");
+            L.decay1 = mat1(st, up, m + "w1"); L.decay2 = mat1(st, up, m + "w2"); L.out = mat1(st, up, m + "o");
+            std::vector<float> mu;
+            for (const char *s : {"r", "k", "v", "g", "w"}) { auto a = st.f32(m + "mu." + s); mu.insert(mu.end(), a.begin(), a.end()); }
+            L.mu = up.vec(mu);
+            L.decay0 = up.vec(st.f32(m + "w0")); L.bonus = up.vec(st.f32(m + "u")); L.onorm = up.vec(st.f32(m + "norm"));
+        } else if (kind == "delta") {
+            L.kind = PS_MIX_DELTA;
+            L.kv_heads = (int32_t)mc.at("kv_heads").num; L.vdim = (int32_t)mc.at("vdim").num; L.conv_taps = (int32_t)mc.at("conv").num;
+            L.in_cat = mat_rows(st, up, {m + "q", m + "k", m + "v", m + "g", m + "b", m + "a"});
+            std::vector<float> cw;
+            for (const char *s : {"q", "k", "v"}) { auto a = expect(st, m + s + ".conv", rows_of(st, m + s), L.conv_taps); cw.insert(cw.end(), a.begin(), a.end()); }
+            L.conv = up.vec(cw);
+            L.a_log = up.vec(st.f32(m + "A_log")); L.dt_bias = up.vec(st.f32(m + "dt_bias")); L.onorm = up.vec(st.f32(m + "norm"));
+            L.out = mat1(st, up, m + "o");
+        } else if (kind == "latent_attention") {
+            L.kind = PS_MIX_LATENT;
+            L.vdim = (int32_t)mc.at("vdim").num; L.q_rank = (int32_t)mc.at("q_rank").num; L.kv_rank = (int32_t)mc.at("kv_rank").num;
+            L.rot_dim = (int32_t)mc.at("rot_dim").num; L.rot_dims = (int32_t)mc.at("rot").at("dims").num; L.rot_base = (float)mc.at("rot").at("base").num;
+            L.window = (int32_t)mc.at("mask").at("size").num; L.scale = (float)mc.at("scale").num;
+            L.in_cat = mat_rows(st, up, {m + "dq", m + "dkv"});
+            L.uq = mat1(st, up, m + "uq");
+            L.ukv = mat_rows(st, up, {m + "uk", m + "uv"});
+            L.out = mat1(st, up, m + "o");
+            L.qnorm = up.vec(st.f32(m + "dq.norm")); L.kvnorm = up.vec(st.f32(m + "dkv.norm"));
+        } else {
+            POWERSERVE_ABORT("layer " + std::to_string(i) + ": mixer type " + kind + " is not known");
+        }
+        layers.push_back(L);
+    }
+}
+} // namespace
+
+const std::map<std::string, SeqArchitecture> &seq_architectures() {
+    static const std::map<std::string, SeqArchitecture> reg = {{"Ranutar", ranutar}};
+    return reg;
+}
+bool is_seq_model_dir(const std::string &dir) {
+    struct stat a, b;
+    return stat((dir + "/config.json").c_str(), &a) == 0 && stat((dir + "/model.safetensors").c_str(), &b) == 0;
+}
+
+// ---------------------------------------------------------------- the model
+SeqModel::SeqModel(const std::string &model_dir, const std::string &dtype, int device, size_t max_batch, int n_slots) {
+    if (dtype != "bfloat16" && dtype != "float32") POWERSERVE_ABORT("dtype " + dtype + ": bfloat16 or float32");
+    JsonValue cfg;
+    try { cfg = JsonValue::parse_file(model_dir + "/config.json"); } catch (const std::exception &e) { POWERSERVE_ABORT(std::string("config.json: ") + e.what()); }
+    if (!cfg.contains("architecture") || !seq_architectures().count(cfg.at("architecture").str))
+        POWERSERVE_ABORT("unknown model type: " + (cfg.contains("architecture") ? cfg.at("architecture").str : std::string("(config.json names no architecture)")));
+    arch = cfg.at("architecture").str;
+    SafeTensorsFile st(model_dir + "/model.safetensors");
+    if (ps_hip_create(device, &m_ctx) != 0) POWERSERVE_ABORT("no HIP device: the MI355X backend cannot run (there is no CPU fallback)");
+    m_up = SeqUploader{m_ctx, dtype == "float32", {}, {}};
+    std::vector<ps_seq_layer> layers;
+    ps_seq_desc d{};
+    try {
+        seq_architectures().at(arch)(cfg, st, m_up, layers, d);
+    } catch (const std::out_of_range &) { POWERSERVE_ABORT("config.json: a tensor has fewer dimensions than its use needs"); }
+    d.n_layers = (int32_t)layers.size();
+    d.max_batch = (int32_t)max_batch;
+    d.n_slots = n_slots;
+    d.compute = dtype == "float32";
+    d.layers = layers.data();
+    hip_ok(m_ctx, ps_hip_seq_create(m_ctx, &d, &m_h), "ps_hip_seq_create");
+    vocab = (uint32_t)d.vocab; width = (uint32_t)d.width; n_layers = (uint32_t)d.n_layers;
+}
+SeqModel::~SeqModel() {
+    if (m_h) ps_hip_seq_destroy(m_h);
+    if (m_ctx) { m_up.free_all(); ps_hip_destroy(m_ctx); }
+}
+int SeqModel::acquire() { int s = -1; hip_ok(m_ctx, ps_hip_seq_acquire(m_h, &s), "ps_hip_seq_acquire"); return s; }
+void SeqModel::release(int slot) { hip_ok(m_ctx, ps_hip_seq_release(m_h, slot), "ps_hip_seq_release"); }
+int64_t SeqModel::position(int slot) const { return ps_hip_seq_position(m_h, slot); }
+std::vector<float> SeqModel::forward(int slot, const std::vector<Token> &tokens, const std::vector<int> &want) {
+    std::vector<float> out(want.size() * (size_t)vocab);
+    hip_ok(m_ctx, ps_hip_seq_forward(m_h, slot, tokens.data(), (int)tokens.size(), want.empty() ? nullptr : want.data(), (int)want.size(),
+                                     want.empty() ? nullptr : out.data(), nullptr), "ps_hip_seq_forward");
+    return out;
+}
+std::vector<Token> SeqModel::generate(const std::vector<Token> &prompt, int steps) {
+    POWERSERVE_ASSERT(!prompt.empty());
+    const int slot = acquire();
+    std::vector<Token> out((size_t)std::max(steps, 0));
+    try {
+        if (prompt.size() > 1) forward(slot, std::vector<Token>(prompt.begin(), prompt.end() - 1), {});
+        hip_ok(m_ctx, ps_hip_seq_decode_greedy(m_h, slot, prompt.back(), steps, out.data()), "ps_hip_seq_decode_greedy");
+    } catch (...) { release(slot); throw; }
+    release(slot);
+    return out;
+}
+std::vector<Token> SeqModel::generate(const std::vector<Token> &prompt, int steps, SamplerChain &sampler) {
+    POWERSERVE_ASSERT(!prompt.empty());
+    const int slot = acquire();
+    std::vector<Token> out;
+    try {
+        if (prompt.size() > 1) forward(slot, std::vector<Token>(prompt.begin(), prompt.end() - 1), {});
+        Token tok = prompt.back();
+        for (int i = 0; i < steps; i++) {
+            auto lg = forward(slot, {tok}, {0});
+            tok = sampler.sample(std::span<const float>(lg.data(), lg.size()));
+            out.push_back(tok);
+        }
+    } catch (...) { release(slot); throw; }
+    release(slot);
+    return out;
+}
+auto load_seq_model(const std::string &model_dir, const std::string &dtype, int device, size_t max_batch, int n_slots) -> std::shared_ptr<SeqModel> {
+    if (!is_seq_model_dir(model_dir)) POWERSERVE_ABORT(model_dir + ": config.json + model.safetensors expected");
+    return std::make_shared<SeqModel>(model_dir, dtype, device, max_batch, n_slots);
+}
+
+} // namespace powerserve
+
+// ---------------------------------------------------------------- C driver API
+using namespace powerserve;
+extern "C" {
+void psh_set_error(const char *msg);
+void *psh_sampler_create(const void *cfg);
+void psh_sampler_free(void *s);
+int psh_is_seq_model_dir(const char *dir) { return is_seq_model_dir(dir) ? 1 : 0; }
+void *psh_seq_load(const char *model_dir, const char *dtype, int device, int max_batch, int n_slots) {
+    try { return new std::shared_ptr<SeqModel>(load_seq_model(model_dir, dtype, device, (size_t)max_batch, n_slots)); } catch (const std::exception &e) { psh_set_error(e.what()); return nullptr; }
+}
+void psh_seq_free(void *h) { delete (std::shared_ptr<SeqModel> *)h; }
+uint32_t psh_seq_vocab(void *h) { return (*(std::shared_ptr<SeqModel> *)h)->vocab; }
+int psh_seq_generate(void *h, const int32_t *prompt, int n_prompt, int steps, int32_t *out) {
+    try {
+        auto r = (*(std::shared_ptr<SeqModel> *)h)->generate(std::vector<Token>(prompt, prompt + n_prompt), steps);
+        memcpy(out, r.data(), r.size() * 4);
+        return 0;
+    } catch (const std::exception &e) { psh_set_error(e.what()); return 1; }
+}
+int psh_seq_generate_sampled(void *h, const int32_t *prompt, int n_prompt, int steps, const void *sampler_cfg, int32_t *out) {
+    void *s = psh_sampler_create(sampler_cfg);
+    if (!s) return 1;
+    int rc = 0;
+    try {
+        auto r = (*(std::shared_ptr<SeqModel> *)h)->generate(std::vector<Token>(prompt, prompt + n_prompt), steps, *(SamplerChain *)s);
+        memcpy(out, r.data(), r.size() * 4);
+    } catch (const std::exception &e) { psh_set_error(e.what()); rc = 1; }
+    psh_sampler_free(s);
+    return rc;
+}
+int psh_seq_forward(void *h, int slot, const int32_t *tokens, int n, const int32_t *want, int n_want, float *logits_out) {
+    try {
+        auto &m = *(std::shared_ptr<SeqModel> *)h;
+        auto r = m->forward(slot, std::vector<Token>(tokens, tokens + n), std::vector<int>(want, want + n_want));
+        if (n_want) memcpy(logits_out, r.data(), r.size() * 4);
+        return 0;
+    } catch (const std::exception &e) { psh_set_error(e.what()); return 1; }
+}
+int psh_seq_acquire(void *h) { try { return (*(std::shared_ptr<SeqModel> *)h)->acquire(); } catch (const std::exception &e) { psh_set_error(e.what()); return -1; } }
+int psh_seq_release(void *h, int slot) { try { (*(std::shared_ptr<SeqModel> *)h)->release(slot); return 0; } catch (const std::exception &e) { psh_set_error(e.what()); return 1; } }
+}

@@ -162,7 +162,28 @@ void psk_boundary1(hipStream_t st, const ps_seq_step *step, float *x, const floa
 typedef float sq_f4 __attribute__((ext_vector_type(4)));
 #define SQ_NR 16 // state rows per lane (lane s of a column holds rows 16 s .. 16 s + 15: its per-token vectors are four 16-byte LDS reads each)
 #define SQ_TC 8  // tokens staged per round
+#define SQ_PF 8  // staged numbers per thread and vector: SQ_TC * 16 R / 256 <= 8 for R <= 16
 static inline int sq_lanes_per_col(int d) { int R = 1; while (R * SQ_NR < d) R *= 2; return R; }
+
+
+// sum over the R (1, 2, 4, 8 or 16) adjacent lanes of a column, every lane gets the total: data-parallel-primitive moves inside a row of 16
+// lanes (neighbour, other pair, mirrored half, mirrored row) instead of trips through the LDS crossbar
+static __device__ __forceinline__ float sq_dpp(float v, int ctrl_sel) {
+    const int x = __float_as_int(v);
+    int y;
+    if (ctrl_sel == 0) y = __builtin_amdgcn_update_dpp(0, x, 0xB1, 0xF, 0xF, false);       // quad_perm [1, 0, 3, 2]
+    else if (ctrl_sel == 1) y = __builtin_amdgcn_update_dpp(0, x, 0x4E, 0xF, 0xF, false);  // quad_perm [2, 3, 0, 1]
+    else if (ctrl_sel == 2) y = __builtin_amdgcn_update_dpp(0, x, 0x141, 0xF, 0xF, false); // row_half_mirror
+    else y = __builtin_amdgcn_update_dpp(0, x, 0x140, 0xF, 0xF, false);                    // row_mirror
+    return __int_as_float(y);
+}
+static __device__ __forceinline__ float sq_col_sum(float v, int R) {
+    if (R > 1) v += sq_dpp(v, 0);
+    if (R > 2) v += sq_dpp(v, 1);
+    if (R > 4) v += sq_dpp(v, 2);
+    if (R > 8) v += sq_dpp(v, 3);
+    return v;
+}
 
 // LDS: rs, ks, ws [TC][dp] (dp = NR * R, rows >= d zero), sc [TC] (sum_i r_i bonus_i k_i)
 __global__ __launch_bounds__(256) void sq_wkv_scan_kernel(const ps_seq_step *step, long long state_off, const float *r, const float *k, const float *v, const float *z,
@@ -180,26 +201,40 @@ __global__ __launch_bounds__(256) void sq_wkv_scan_kernel(const ps_seq_step *ste
         S[m] = (col && i < d) ? S0[(long long)i * d + j] : 0.f;
     }
     const long long hb = (long long)h * d;
+    // the next round's inputs are requested before the current round's steps run, and land in LDS after them
+    float pa[SQ_PF], pb[SQ_PF], pc[SQ_PF], pv[SQ_TC];
+    auto fetch = [&](int t0) {
+        const int nt = min(SQ_TC, T - t0);
+#pragma unroll
+        for (int e = 0; e < SQ_PF; e++) {
+            const int x = tid + 256 * e, t = x / dp, i = x % dp;
+            const bool in = x < SQ_TC * dp && t < nt && i < d;
+            const long long at = (long long)(t0 + (in ? t : 0)) * ld + hb + (in ? i : 0);
+            pa[e] = in ? r[at] : 0.f;
+            pb[e] = in ? k[at] : 0.f;
+            pc[e] = in ? z[at] : INFINITY; // exp(-exp(inf)) = 0
+        }
+#pragma unroll
+        for (int t = 0; t < SQ_TC; t++) pv[t] = (col && t < nt) ? v[(long long)(t0 + t) * ld + hb + j] : 0.f;
+    };
+    fetch(0);
     for (int t0 = 0; t0 < T; t0 += SQ_TC) {
         const int nt = min(SQ_TC, T - t0);
         __syncthreads();
-        for (int x = tid; x < SQ_TC * dp; x += 256) {
-            const int t = x / dp, i = x % dp;
-            float a = 0.f, b = 0.f, c = 0.f;
-            if (t < nt && i < d) {
-                const long long at = (long long)(t0 + t) * ld + hb + i;
-                a = r[at];
-                b = k[at];
-                c = expf(-expf(z[at]));
+#pragma unroll
+        for (int e = 0; e < SQ_PF; e++) {
+            const int x = tid + 256 * e;
+            if (x < SQ_TC * dp) {
+                rs[x] = pa[e];
+                ks[x] = pb[e];
+                ws[x] = expf(-expf(pc[e]));
             }
-            rs[x] = a;
-            ks[x] = b;
-            ws[x] = c;
         }
         float vj[SQ_TC];
 #pragma unroll
-        for (int t = 0; t < SQ_TC; t++) vj[t] = (col && t < nt) ? v[(long long)(t0 + t) * ld + hb + j] : 0.f;
+        for (int t = 0; t < SQ_TC; t++) vj[t] = pv[t];
         __syncthreads();
+        if (t0 + SQ_TC < T) fetch(t0 + SQ_TC);
         for (int t = tid >> 6; t < SQ_TC; t += 4) { // one wave per token
             float a = 0.f;
             for (int i = tid & 63; i < d; i += 64) a += rs[t * dp + i] * bonus[hb + i] * ks[t * dp + i];
@@ -212,17 +247,17 @@ __global__ __launch_bounds__(256) void sq_wkv_scan_kernel(const ps_seq_step *ste
         for (int t = 0; t < SQ_TC; t++) {
             if (t < nt) {
                 const sq_f4 *rt = (const sq_f4 *)(rs + t * dp + s * SQ_NR), *kt = (const sq_f4 *)(ks + t * dp + s * SQ_NR), *wt = (const sq_f4 *)(ws + t * dp + s * SQ_NR);
-                float p = 0.f;
+                float pp[4] = {0.f, 0.f, 0.f, 0.f}; // four short chains instead of one of sixteen
 #pragma unroll
                 for (int m4 = 0; m4 < SQ_NR / 4; m4++) {
                     const sq_f4 r4 = rt[m4], k4 = kt[m4], w4 = wt[m4];
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
-                        p = fmaf(r4[e], S[4 * m4 + e], p);
+                        pp[e] = fmaf(r4[e], S[4 * m4 + e], pp[e]);
                         S[4 * m4 + e] = fmaf(w4[e], S[4 * m4 + e], k4[e] * vj[t]);
                     }
                 }
-                for (int x = 1; x < R; x <<= 1) p += __shfl_xor(p, x, 64);
+                const float p = sq_col_sum((pp[0] + pp[1]) + (pp[2] + pp[3]), R);
                 if (col && s == 0) o[(long long)(t0 + t) * ldo + hb + j] = fmaf(vj[t], sc[t], p);
             }
         }
@@ -259,24 +294,46 @@ __global__ __launch_bounds__(256) void sq_delta_scan_kernel(const ps_seq_step *s
     }
     const long long qb = (long long)(h / (H / KH)) * d, vb = (long long)h * dv;
     const float qscale = 1.f / sqrtf((float)d), na = -expf(a_log[h]), db = dt_bias[h];
-    for (int t0 = 0; t0 < T; t0 += SQ_TC) {
+    float pa[SQ_PF], pb[SQ_PF], pv[SQ_TC], pg = 0.f, pbeta = 0.f;
+    auto fetch = [&](int t0) {
         const int nt = min(SQ_TC, T - t0);
-        __syncthreads();
-        for (int x = tid; x < SQ_TC * dp; x += 256) {
-            const int t = x / dp, i = x % dp;
-            const bool in = t < nt && i < d;
-            qs[x] = in ? q[(long long)(t0 + t) * ld + qb + i] : 0.f;
-            ks[x] = in ? k[(long long)(t0 + t) * ld + qb + i] : 0.f;
+#pragma unroll
+        for (int e = 0; e < SQ_PF; e++) {
+            const int x = tid + 256 * e, t = x / dp, i = x % dp;
+            const bool in = x < SQ_TC * dp && t < nt && i < d;
+            const long long at = (long long)(t0 + (in ? t : 0)) * ld + qb + (in ? i : 0);
+            pa[e] = in ? q[at] : 0.f;
+            pb[e] = in ? k[at] : 0.f;
         }
         if (tid < SQ_TC) {
             const bool in = tid < nt;
-            gs[tid] = in ? expf(na * sq_softplus(araw[(long long)(t0 + tid) * ldb + h] + db)) : 1.f;
-            bs[tid] = in ? 1.f / (1.f + expf(-braw[(long long)(t0 + tid) * ldb + h])) : 0.f;
+            pg = in ? araw[(long long)(t0 + tid) * ldb + h] : 0.f;
+            pbeta = in ? braw[(long long)(t0 + tid) * ldb + h] : -INFINITY; // sigmoid(-inf) = 0
+        }
+#pragma unroll
+        for (int t = 0; t < SQ_TC; t++) pv[t] = (col && t < nt) ? v[(long long)(t0 + t) * ld + vb + j] : 0.f;
+    };
+    fetch(0);
+    for (int t0 = 0; t0 < T; t0 += SQ_TC) {
+        const int nt = min(SQ_TC, T - t0);
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < SQ_PF; e++) {
+            const int x = tid + 256 * e;
+            if (x < SQ_TC * dp) {
+                qs[x] = pa[e];
+                ks[x] = pb[e];
+            }
+        }
+        if (tid < SQ_TC) {
+            gs[tid] = tid < nt ? expf(na * sq_softplus(pg + db)) : 1.f;
+            bs[tid] = 1.f / (1.f + expf(-pbeta));
         }
         float vj[SQ_TC];
 #pragma unroll
-        for (int t = 0; t < SQ_TC; t++) vj[t] = (col && t < nt) ? v[(long long)(t0 + t) * ld + vb + j] : 0.f;
+        for (int t = 0; t < SQ_TC; t++) vj[t] = pv[t];
         __syncthreads();
+        if (t0 + SQ_TC < T) fetch(t0 + SQ_TC);
         for (int t = tid >> 6; t < SQ_TC; t += 4) { // one wave per token: unit vectors, then k . q
             float a = 0.f, b = 0.f;
             for (int i = tid & 63; i < d; i += 64) {
@@ -307,7 +364,7 @@ __global__ __launch_bounds__(256) void sq_delta_scan_kernel(const ps_seq_step *s
                 const sq_f4 *qt = (const sq_f4 *)(qs + t * dp + s * SQ_NR), *kt = (const sq_f4 *)(ks + t * dp + s * SQ_NR);
                 const float g = gs[t];
                 sq_f4 k4[SQ_NR / 4];
-                float p1 = 0.f, p2 = 0.f;
+                float a1[4] = {0.f, 0.f, 0.f, 0.f}, a2[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int m4 = 0; m4 < SQ_NR / 4; m4++) {
                     const sq_f4 q4 = qt[m4];
@@ -315,14 +372,11 @@ __global__ __launch_bounds__(256) void sq_delta_scan_kernel(const ps_seq_step *s
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
                         S[4 * m4 + e] *= g;
-                        p1 = fmaf(k4[m4][e], S[4 * m4 + e], p1);
-                        p2 = fmaf(q4[e], S[4 * m4 + e], p2);
+                        a1[e] = fmaf(k4[m4][e], S[4 * m4 + e], a1[e]);
+                        a2[e] = fmaf(q4[e], S[4 * m4 + e], a2[e]);
                     }
                 }
-                for (int x = 1; x < R; x <<= 1) {
-                    p1 += __shfl_xor(p1, x, 64);
-                    p2 += __shfl_xor(p2, x, 64);
-                }
+                const float p1 = sq_col_sum((a1[0] + a1[1]) + (a1[2] + a1[3]), R), p2 = sq_col_sum((a2[0] + a2[1]) + (a2[2] + a2[3]), R);
                 const float u = bs[t] * (vj[t] - p1);
 #pragma unroll
                 for (int m4 = 0; m4 < SQ_NR / 4; m4++)

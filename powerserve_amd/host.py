@@ -12,6 +12,7 @@ LIB_PATH = os.path.join(HERE, "lib", "libps_host.so")
 EXPORTS = ["psh_last_error", "psh_model_load", "psh_model_free", "psh_model_set_fused", "psh_model_plan_stats", "psh_model_kv_position", "psh_model_reset",
            "psh_model_vocab", "psh_model_forward", "psh_model_generate", "psh_spec_generate", "psh_spec_generate_sampled", "psh_draft_sample", "psh_sampler_create", "psh_sampler_free", "psh_sampler_sample",
            "psh_model_generate_sampled", "psh_token_tree_run", "psh_gguf_summary", "psh_config_summary",
+           "psh_is_seq_model_dir", "psh_seq_load", "psh_seq_free", "psh_seq_vocab", "psh_seq_generate", "psh_seq_generate_sampled", "psh_seq_forward", "psh_seq_acquire", "psh_seq_release",
            "psh_model_decode", "psh_model_prefill", "psh_model_plan_cache_hits", "psh_model_set_plan_cache", "psh_graph_softmax", "psh_backend_get_n_tasks", "psh_backend_add_cache", "psh_model_kv_read", "psh_kv_op"]
 _LIB = None
 
@@ -55,6 +56,17 @@ def lib() -> C.CDLL:
         L.psh_model_kv_read.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_void_p, C.c_void_p]
         L.psh_kv_op.restype = C.c_int64
         L.psh_kv_op.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_int64]
+        L.psh_is_seq_model_dir.argtypes = [C.c_char_p]
+        L.psh_seq_load.restype = C.c_void_p
+        L.psh_seq_load.argtypes = [C.c_char_p, C.c_char_p, C.c_int, C.c_int, C.c_int]
+        L.psh_seq_free.argtypes = [C.c_void_p]
+        L.psh_seq_vocab.restype = C.c_uint32
+        L.psh_seq_vocab.argtypes = [C.c_void_p]
+        L.psh_seq_generate.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
+        L.psh_seq_generate_sampled.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+        L.psh_seq_forward.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_void_p]
+        L.psh_seq_acquire.argtypes = [C.c_void_p]
+        L.psh_seq_release.argtypes = [C.c_void_p, C.c_int]
         L.psh_config_summary.restype = C.c_int64
         L.psh_config_summary.argtypes = [C.c_char_p, C.c_char_p, C.c_size_t]
         L.psh_gguf_summary.restype = C.c_int64
@@ -398,3 +410,48 @@ class Workspace:
         self.main.close()
         if self.draft is not None:
             self.draft.close()
+
+
+class HostSeqModel:
+    """load_seq_model(dir) of the C++ facade (csrc/host/seq_model.cpp): a layer-list model from config.json + model.safetensors."""
+
+    def __init__(self, model_dir: str, dtype: str = "bfloat16", device: int = 0, max_batch: int = 256, n_slots: int = 2):
+        self.L = lib()
+        self.h = self.L.psh_seq_load(model_dir.encode(), dtype.encode(), device, max_batch, n_slots)
+        if not self.h:
+            raise HostError(self.L.psh_last_error().decode())
+        self.vocab = int(self.L.psh_seq_vocab(self.h))
+
+    def close(self):
+        if getattr(self, "h", None):
+            self.L.psh_seq_free(self.h)
+            self.h = None
+
+    def _check(self, rc):
+        if rc != 0:
+            raise HostError(self.L.psh_last_error().decode())
+
+    def generate(self, prompt, steps: int, sampler_cfg: SamplerCfg | None = None) -> np.ndarray:
+        p = np.ascontiguousarray(prompt, dtype=np.int32)
+        out = np.empty(steps, dtype=np.int32)
+        if sampler_cfg is None:
+            self._check(self.L.psh_seq_generate(self.h, p.ctypes.data, p.size, steps, out.ctypes.data))
+        else:
+            self._check(self.L.psh_seq_generate_sampled(self.h, p.ctypes.data, p.size, steps, C.byref(sampler_cfg), out.ctypes.data))
+        return out
+
+    def forward(self, slot: int, tokens, want) -> np.ndarray:
+        t = np.ascontiguousarray(tokens, dtype=np.int32)
+        w = np.ascontiguousarray(want, dtype=np.int32)
+        out = np.empty((w.size, self.vocab), dtype=np.float32)
+        self._check(self.L.psh_seq_forward(self.h, slot, t.ctypes.data, t.size, w.ctypes.data, w.size, out.ctypes.data))
+        return out
+
+    def acquire(self) -> int:
+        s = self.L.psh_seq_acquire(self.h)
+        if s < 0:
+            raise HostError(self.L.psh_last_error().decode())
+        return s
+
+    def release(self, slot: int):
+        self._check(self.L.psh_seq_release(self.h, slot))

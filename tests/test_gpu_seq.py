@@ -292,6 +292,26 @@ def test_matrix_core_forms_agree_with_the_plain_kernels(made, dtype):
         assert err(a, want) < TOL[dtype]
 
 
+def test_host_facade_loads_and_generates_the_same(made, tmp_path):
+    """load_seq_model of the C++ facade (its own safetensors reader and configuration mapping) over the same files: same ids, same logits"""
+    m, cfg, t = made("mixed", "float32", max_batch=16)
+    synth.write_seq_model_dir(str(tmp_path), cfg, 0, t)
+    assert host.lib().psh_is_seq_model_dir(str(tmp_path).encode()) == 1
+    hm = host.HostSeqModel(str(tmp_path), dtype="float32", max_batch=16, n_slots=2)
+    prompt = tokens_for(cfg, 19, seed=7)
+    ids = m.generate(prompt, 12)
+    assert np.array_equal(hm.generate(prompt, 12), ids)
+    assert np.array_equal(hm.generate(prompt, 12, host.SamplerCfg.make(cfg["vocab"], seed=3, temperature=1.0, top_p=1.0, top_k=1)), ids)
+    s, s2 = hm.acquire(), m.acquire()
+    a, b = hm.forward(s, prompt, [0, 5, 18]), m.forward(s2, prompt, [0, 5, 18])
+    hm.release(s)
+    m.release(s2)
+    assert np.array_equal(a, b)
+    with pytest.raises(host.HostError):
+        host.HostModel(str(tmp_path))  # the quantized path's loader says what this folder is instead of looking for model.json
+    hm.close()
+
+
 def test_refusals(ctx, tmp_path):
     cfg = dict(CONFIGS["wkv"])
     synth.write_seq_model_dir(str(tmp_path), cfg, 0)
