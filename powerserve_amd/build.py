@@ -30,6 +30,11 @@ SEQ_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 NOSLP = {"k_gemv4.hip", "k_qkvattn.hip", "k_gemvb.hip", "k_attn.hip", "k_gemm4k.hip"}  # k_gemm4k.hip (round 5): gate/up chunk launch of a 512-column sequence 384.2 -> 369-371 us, same bits (profiles/r05_g4k2_variants.txt, the "v2 0" lines vs profiles/r05_g4k_item_order.txt)  # (k_gemvb.hip: the Q4_0 / Q8_0 mat-vec, Llama-3.2-1B 1494 -> 1525 tok/s)
 
 
+def _stale(so: str, objs: list) -> bool:
+    """the library is missing or older than one of its objects (the two libraries share objects: what one build compiled the other must still link)"""
+    return not os.path.exists(so) or any(os.path.getmtime(o) > os.path.getmtime(so) for o in objs)
+
+
 def _cmd_changed(obj: str, cmd: list) -> bool:
     """the exact compile command is kept next to the object: an edited flag list rebuilds it (mtimes alone let stale objects survive)"""
     try:
@@ -83,7 +88,7 @@ def build_seq(force: bool = False, verbose: bool = True) -> str:
     with ThreadPoolExecutor(max_workers=8) as ex:
         list(ex.map(run, jobs))
     so = os.path.join(LIBDIR, "libps_hip_seq.so")
-    if jobs or not os.path.exists(so):
+    if jobs or _stale(so, objs):
         tmp = so + ".%d.tmp" % os.getpid()
         subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs], check=True)
         os.replace(tmp, so)
@@ -127,10 +132,10 @@ def build(force: bool = False, verbose: bool = True, contract: bool = True, time
     with ThreadPoolExecutor(max_workers=8) as ex:
         list(ex.map(run, jobs))
     so = os.path.join(LIBDIR, "libps_hip.so")
-    if jobs or not os.path.exists(so):
+    if jobs or _stale(so, objs):
         subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", so, *objs], check=True)
     cso = os.path.join(LIBDIR, "libps_hip_contract.so")
-    if contract and (jobs or not os.path.exists(cso)):
+    if contract and (jobs or _stale(cso, cobjs)):
         subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", cso, *cobjs], check=True)
     tso = os.path.join(LIBDIR, "libps_hip_timeline.so")
     if not timeline and jobs and os.path.exists(tso):
