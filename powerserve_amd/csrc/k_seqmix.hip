@@ -212,7 +212,7 @@ __global__ __launch_bounds__(256) void sq_wkv_scan_kernel(const ps_seq_step *ste
             const long long at = (long long)(t0 + (in ? t : 0)) * ld + hb + (in ? i : 0);
             pa[e] = in ? r[at] : 0.f;
             pb[e] = in ? k[at] : 0.f;
-            pc[e] = in ? z[at] : INFINITY; // exp(-exp(inf)) = 0
+            pc[e] = in ? z[at] : -INFINITY; // exp(-exp(-inf)) = 1: with k = 0 a token that is not there leaves the state alone
         }
 #pragma unroll
         for (int t = 0; t < SQ_TC; t++) pv[t] = (col && t < nt) ? v[(long long)(t0 + t) * ld + hb + j] : 0.f;
@@ -243,9 +243,10 @@ __global__ __launch_bounds__(256) void sq_wkv_scan_kernel(const ps_seq_step *ste
             if ((tid & 63) == 0) sc[t] = a;
         }
         __syncthreads();
+        // (no branch per token: the steps of a round are one block of straight-line code the compiler can interleave; padded tokens are neutral)
 #pragma unroll
         for (int t = 0; t < SQ_TC; t++) {
-            if (t < nt) {
+            {
                 const sq_f4 *rt = (const sq_f4 *)(rs + t * dp + s * SQ_NR), *kt = (const sq_f4 *)(ks + t * dp + s * SQ_NR), *wt = (const sq_f4 *)(ws + t * dp + s * SQ_NR);
                 float pp[4] = {0.f, 0.f, 0.f, 0.f}; // four short chains instead of one of sixteen
 #pragma unroll
@@ -258,7 +259,7 @@ __global__ __launch_bounds__(256) void sq_wkv_scan_kernel(const ps_seq_step *ste
                     }
                 }
                 const float p = sq_col_sum((pp[0] + pp[1]) + (pp[2] + pp[3]), R);
-                if (col && s == 0) o[(long long)(t0 + t) * ldo + hb + j] = fmaf(vj[t], sc[t], p);
+                if (col && s == 0 && t < nt) o[(long long)(t0 + t) * ldo + hb + j] = fmaf(vj[t], sc[t], p);
             }
         }
     }
@@ -360,7 +361,7 @@ __global__ __launch_bounds__(256) void sq_delta_scan_kernel(const ps_seq_step *s
         __syncthreads();
 #pragma unroll
         for (int t = 0; t < SQ_TC; t++) {
-            if (t < nt) {
+            { // (padded tokens: g = 1, beta = 0, k = 0 -- the state stays)
                 const sq_f4 *qt = (const sq_f4 *)(qs + t * dp + s * SQ_NR), *kt = (const sq_f4 *)(ks + t * dp + s * SQ_NR);
                 const float g = gs[t];
                 sq_f4 k4[SQ_NR / 4];
@@ -382,7 +383,7 @@ __global__ __launch_bounds__(256) void sq_delta_scan_kernel(const ps_seq_step *s
                 for (int m4 = 0; m4 < SQ_NR / 4; m4++)
 #pragma unroll
                     for (int e = 0; e < 4; e++) S[4 * m4 + e] = fmaf(k4[m4][e], u, S[4 * m4 + e]);
-                if (col && s == 0) o[(long long)(t0 + t) * ldo + vb + j] = fmaf(u, kq[t], p2); // S_new^T q = (g S)^T q + u (k . q)
+                if (col && s == 0 && t < nt) o[(long long)(t0 + t) * ldo + vb + j] = fmaf(u, kq[t], p2); // S_new^T q = (g S)^T q + u (k . q)
             }
         }
     }
