@@ -1,8 +1,9 @@
 // Dense (unquantized) matrices of the layer-list models: bfloat16 operands with fp32 accumulation on v_mfma_f32_16x16x32_bf16, or
 // fp32 throughout on v_mfma_f32_16x16x4_f32 (one rounding per product, fp32 adds: a true fp32 product, no reduced-precision mode).
 //   dense_mm_kernel<WT>   tiled mat-mul, 64 tokens x 64 outputs per work-group of four waves, any T / N / K (edges zero-filled)
+//   dense_mm_fast_kernel  bf16, K % 64 == 0, more than 8 tokens: 128 x 128 tiles over an operand packed to bf16 by dense_pack_kernel
 //   dense_mv_kernel<WT,C> a few tokens (C <= 8 columns): the activation rows live in LDS, a wave streams four weight rows at a time
-// Both take the same operand description (ps_seq.h psk_dense_args): ring rows, the token-shift mix and the epilogue
+// All take the same operand description (ps_seq.h psk_dense_args): ring rows, the token-shift mix and the epilogue
 // (bias, xIELU / tanh, scale) are part of the launch, so no mixer needs a kernel of its own around its projections.
 #include "ps_seq.h"
 

@@ -3,6 +3,7 @@
 // widest step, so a step never overwrites a row one of its own tokens still sees).  Scores, soft-max and the weighted sum are fp32.
 //   latent_prep_kernel   norms of the two latents, rotation of the shared key part, ring append
 //   latent_attn_kernel   one wave per (token, head) over per-head keys / values expanded from the ring rows of the window (the plain form)
+//   latent_attn_mfma_kernel / latent_absorbed_kernel (+ fold, combine, unfold): the matrix-core forms for a portion and for a single token, below
 #include "ps_seq.h"
 
 #include <cmath>

@@ -53,7 +53,7 @@ void psk_norm_residual(hipStream_t st, float *x, const float *y, const float *w,
 }
 
 // ---------------------------------------------------------------------------------------------------- causal convolution with a tail
-#define SQ_CONV_CHUNK 32
+#define SQ_CONV_CHUNK 8 // tokens per thread: a portion spreads over T / 8 times as many threads as channels
 static __device__ __forceinline__ void sq_conv_tail(float *tail, const float *in, long long ldi, int taps, long long C, int T, long long c) {
     // new tail row i = input of token T - (taps-1) + i; before this step's first token: the old tail's row T + i (ascending i never reads a row already written)
     for (int i = 0; i < taps - 1; i++) {

@@ -248,6 +248,8 @@ class RequestScheduler:
     def feed(self, rid, tokens, want=None) -> np.ndarray:
         if rid not in self.slots:
             self.slots[rid] = self.model.acquire()
+        if len(tokens) == 0:
+            return np.empty((0, self.model.vocab), dtype=np.float32)
         return self.model.forward(self.slots[rid], tokens, want)
 
     def finish(self, rid):
