@@ -248,20 +248,20 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const ps_seq_step
     if (t0 >= T) return; // (no block-wide barrier below: waves are on their own)
     const long long first = pos0 - window + 1 > 0 ? pos0 - window + 1 : 0;
     const int half = rot_dims / 2;
-    for (int x = lane; x < 16 * (d + dr); x += 64) {
-        const int r = x / (d + dr), c = x % (d + dr), t = t0 + r;
-        float v = 0.f;
-        if (t < T) {
-            const float *qt = q + (long long)t * ldq + (long long)h * (d + dr);
-            v = qt[c];
-            const int cr = c - d;
-            if (cr >= 0 && cr < 2 * half) {
-                const int i = cr < half ? cr : cr - half;
-                const float ang = (float)(pos0 + t) * freq[i], cs = cosf(ang), sn = sinf(ang);
-                v = cr < half ? qt[d + i] * cs - qt[d + half + i] * sn : qt[d + half + i] * cs + qt[d + i] * sn;
-            }
+    // this wave's 16 query rows into LDS (no index division, one sincos per rotated pair and row)
+    for (int r = 0; r < 16; r++) {
+        const int t = t0 + r;
+        const bool in = t < T;
+        const float *qt = q + (long long)(in ? t : 0) * ldq + (long long)h * (d + dr);
+        float *qr = qs + r * qld;
+        for (int c = lane; c < d; c += 64) qr[c] = in ? qt[c] : 0.f;
+        for (int c = 2 * half + lane; c < dr; c += 64) qr[d + c] = in ? qt[d + c] : 0.f;
+        for (int i = lane; i < half; i += 64) {
+            const float ang = (float)(pos0 + t) * freq[i], cs = cosf(ang), sn = sinf(ang);
+            const float u = in ? qt[d + i] : 0.f, v = in ? qt[d + half + i] : 0.f;
+            qr[d + i] = u * cs - v * sn;
+            qr[d + half + i] = v * cs + u * sn;
         }
-        qs[r * qld + c] = v;
     }
     __builtin_amdgcn_wave_barrier();
     const la_src k1 = {kv + (long long)h * d, ldkv, first, 0};
@@ -280,12 +280,13 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const ps_seq_step
 #pragma unroll
     for (int J = 0; J < NJ / 4; J++)
 #pragma unroll
-        for (int jj = 0; jj < 4; jj++)
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int t = t0 + 4 * lq + i, c = 64 * J + 4 * lr + jj;
-                if (t < T && c < dv) o[(long long)t * ldo + (long long)h * dv + c] = acc[4 * J + jj][i] / l[i];
+        for (int i = 0; i < 4; i++) { // a lane's four tiles of a 64-column group are four consecutive columns: one 16-byte store
+            const int t = t0 + 4 * lq + i, c = 64 * J + 4 * lr;
+            if (t < T && c < dv) {
+                const float il = 1.f / l[i];
+                *(la_f4 *)(o + (long long)t * ldo + (long long)h * dv + c) = la_f4{acc[4 * J][i] * il, acc[4 * J + 1][i] * il, acc[4 * J + 2][i] * il, acc[4 * J + 3][i] * il};
             }
+        }
 }
 
 bool psk_latent_attn_mfma_ok(int d, int dr, int dv) { return d % 16 == 0 && dr % 16 == 0 && dv % 4 == 0 && dv <= 128 && (size_t)4 * (16 * (d + dr + 4) + 16 * 17) * 4 <= 160 * 1024; }
@@ -336,8 +337,8 @@ __global__ __launch_bounds__(256) void latent_unfold_v_kernel(const float *ol, c
     if (lane == 0) o[row] = a;
 }
 
-// rows = heads (16 per block), keys = ring rows; wave w of block (split s, head tile) takes key tile 4 s + w of the window.  Partials
-// part[(tile * H16 + ht) ...]: per (key tile, head) m, l and R unnormalised outputs.  dynamic LDS: 16 x qld + 4 x 16 x 17
+// rows = heads (16 per block), keys = ring rows; wave w of block (split s, head tile) takes key tile 4 s + w of the window.  Partials:
+// per (key tile, head) R unnormalised outputs, then m and l.  dynamic LDS: 16 x qld + 4 x 16 x 17
 template <int NJ>
 __global__ __launch_bounds__(256) void latent_absorbed_kernel(const ps_seq_step *step, long long ring_off, int cap, const float *qa, const float *q, int qstride, int d,
                                                               int dr, int rot_dims, const float *freq, int H, int R, int window, float scale, float *part) {
@@ -348,23 +349,22 @@ __global__ __launch_bounds__(256) void latent_absorbed_kernel(const ps_seq_step 
     const long long p = step->pos0;
     const long long lo = p - window + 1 > 0 ? p - window + 1 : 0;
     const int half = rot_dims / 2;
-    for (int x = threadIdx.x; x < 16 * (R + dr); x += 256) {
-        const int r = x / (R + dr), c = x % (R + dr), h = h0 + r;
-        float v = 0.f;
-        if (h < H) {
-            if (c < R) v = qa[(long long)h * R + c];
-            else {
-                const float *qt = q + (long long)h * qstride + d;
-                const int cr = c - R;
-                v = qt[cr];
-                if (cr < 2 * half) {
-                    const int i = cr < half ? cr : cr - half;
-                    const float ang = (float)p * freq[i], cs = cosf(ang), sn = sinf(ang);
-                    v = cr < half ? qt[i] * cs - qt[half + i] * sn : qt[half + i] * cs + qt[i] * sn;
-                }
-            }
+    // the 16 heads' folded queries and rotated parts into LDS: wave w takes rows w, w + 4, ...; every head turns by the same angles
+    for (int r = wave; r < 16; r += 4) {
+        const int h = h0 + r;
+        float *qr = qs + r * qld;
+        for (int c = lane; c < R; c += 64) qr[c] = h < H ? qa[(long long)h * R + c] : 0.f;
+        for (int c = 2 * half + lane; c < dr; c += 64) qr[R + c] = h < H ? q[(long long)h * qstride + d + c] : 0.f;
+    }
+    for (int i = lane; i < half; i += 64) {
+        const float ang = (float)p * freq[i], cs = cosf(ang), sn = sinf(ang);
+        for (int r = wave; r < 16; r += 4) {
+            const int h = h0 + r;
+            const float *qt = q + (long long)(h < H ? h : 0) * qstride + d;
+            const float u = h < H ? qt[i] : 0.f, v = h < H ? qt[half + i] : 0.f;
+            qs[r * qld + R + i] = u * cs - v * sn;
+            qs[r * qld + R + half + i] = v * cs + u * sn;
         }
-        qs[r * qld + c] = v;
     }
     __syncthreads();
     const long long tile = (long long)blockIdx.x * 4 + wave, j0 = lo + tile * 16;
@@ -378,20 +378,18 @@ __global__ __launch_bounds__(256) void latent_absorbed_kernel(const ps_seq_step 
 #pragma unroll
     for (int j = 0; j < NJ; j++) acc[j] = la_f4{0.f, 0.f, 0.f, 0.f};
     if (j0 <= p) la_tile<NJ>(qs, qld, pt, k1, k2, k1, R, dr, R, j0, p + 1, rowpos, window, scale, m, l, acc);
-    // partial of (tile, head): [m, l, o[R]]
+    // partial of (tile, head): [o[R], m, l, -, -] (rows of R + 4 floats: 16-byte stores)
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const int h = h0 + 4 * lq + i;
         if (h >= H) continue;
-        float *pp = part + ((long long)tile * H + h) * (R + 2);
-        if (lr == 0) { pp[0] = m[i]; pp[1] = l[i]; }
+        float *pp = part + ((long long)tile * H + h) * (R + 4);
+        if (lr == 0) { pp[R] = m[i]; pp[R + 1] = l[i]; }
 #pragma unroll
-        for (int J = 0; J < NJ / 4; J++)
-#pragma unroll
-            for (int jj = 0; jj < 4; jj++) {
-                const int c = 64 * J + 4 * lr + jj;
-                if (c < R) pp[2 + c] = acc[4 * J + jj][i];
-            }
+        for (int J = 0; J < NJ / 4; J++) {
+            const int c = 64 * J + 4 * lr;
+            if (c < R) *(la_f4 *)(pp + c) = la_f4{acc[4 * J][i], acc[4 * J + 1][i], acc[4 * J + 2][i], acc[4 * J + 3][i]};
+        }
     }
 }
 // ol[h][c] = sum_tiles exp(m_t - M) o_t[c] / sum_tiles exp(m_t - M) l_t
@@ -403,7 +401,7 @@ __global__ __launch_bounds__(256) void latent_combine_kernel(const ps_seq_step *
     int nt = (int)((p - lo) / 16 + 1);
     if (nt > max_tiles) nt = max_tiles;
     float mx = -INFINITY;
-    for (int t = tid; t < nt; t += 256) mx = fmaxf(mx, part[((long long)t * H + h) * (R + 2)]);
+    for (int t = tid; t < nt; t += 256) mx = fmaxf(mx, part[((long long)t * H + h) * (R + 4) + R]);
     mx = la_wave_max(mx);
     if ((tid & 63) == 0) red[tid >> 6] = mx;
     __syncthreads();
@@ -411,7 +409,7 @@ __global__ __launch_bounds__(256) void latent_combine_kernel(const ps_seq_step *
     __syncthreads();
     float ls = 0.f;
     for (int t = tid; t < nt; t += 256) {
-        const float *pp = part + ((long long)t * H + h) * (R + 2);
+        const float *pp = part + ((long long)t * H + h) * (R + 4) + R;
         const float w = pp[0] == -INFINITY ? 0.f : expf(pp[0] - M);
         wts[t] = w;
         ls = fmaf(w, pp[1], ls);
@@ -422,13 +420,14 @@ __global__ __launch_bounds__(256) void latent_combine_kernel(const ps_seq_step *
     const float L = red[0] + red[1] + red[2] + red[3];
     for (int c = tid; c < R; c += 256) {
         float a = 0.f;
-        for (int t = 0; t < nt; t++) a = fmaf(wts[t], part[((long long)t * H + h) * (R + 2) + 2 + c], a);
+#pragma unroll 8
+        for (int t = 0; t < nt; t++) a = fmaf(wts[t], part[((long long)t * H + h) * (R + 4) + c], a);
         ol[(long long)h * R + c] = a / L;
     }
 }
 
 bool psk_latent_absorbed_ok(int d, int dr, int dv, int R) { return R % 16 == 0 && dr % 16 == 0 && R <= 512 && (size_t)(16 * (R + dr + 4) + 4 * 16 * 17) * 4 <= 160 * 1024; }
-size_t psk_latent_absorbed_scratch(int H, int R, int window) { return ((size_t)((window + 15) / 16 + 4) * H * (R + 2) + (size_t)2 * H * R) * 4; }
+size_t psk_latent_absorbed_scratch(int H, int R, int window) { return ((size_t)((window + 15) / 16 + 4) * H * (R + 4) + (size_t)2 * H * R) * 4; }
 // q [H][d + dr] (row stride qstride) -> o [H * dv]; ukv: rows uk | uv of the expansion matrix [H d + H dv][R]; scratch from psk_latent_absorbed_scratch
 void psk_latent_absorbed(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, const float *q, int qstride, const ps_dense *ukv, const float *freq,
                          int H, int d, int dr, int rot_dims, int dv, int R, int window, float scale, float *scratch, float *o) {
