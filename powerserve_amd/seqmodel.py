@@ -7,7 +7,7 @@ Ranutar: a list of layers, each  x += norm_b(mixer(conv(norm(x))))  and, where i
   wkv               per-channel decayed outer-product state with token-shift mixes and a bonus for the current token
   delta             gated delta rule with short convolutions on q / k / v
   latent_attention  attention over a low-rank latent + one shared rotated key part, sliding window
-the norms RMS with weights stored around zero, the feed-forward dense with the xIELU activation.
+the norms RMS norms whose stored weight is the deviation from one, the feed-forward two dense matrices around the xIELU activation.
 """
 from __future__ import annotations
 
