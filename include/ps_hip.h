@@ -308,8 +308,20 @@ enum ps_mixer_kind {
     PS_MIX_WKV    = 1, /* per-channel decayed outer-product state, token-shift mixes, bonus for the current token */
     PS_MIX_DELTA  = 2, /* gated delta rule: per-head scalar decay, write strength beta, short convolutions on q / k / v */
     PS_MIX_LATENT = 3, /* attention over a low-rank latent + one shared rotated key part, sliding window */
+    PS_MIX_WINATTN = 4, /* grouped-query attention over a sliding window + one mean key / value per block of `pool` tokens wholly before it,
+                         * a sink in the soft-max denominator, a temperature per head, norms over the whole q / k projections, partial rotary, a gate per head */
+    PS_MIX_GLA    = 5, /* gated linear attention: S <- diag(alpha) S + k v^T, o = S^T q, a decay per key channel from a two-matrix projection */
 };
-enum ps_ff_kind { PS_FF_NONE = 0, PS_FF_DENSE_XIELU = 1 };
+enum ps_ff_kind {
+    PS_FF_NONE = 0,
+    PS_FF_DENSE_XIELU = 1,  /* W_down xIELU(W_up h) */
+    PS_FF_DENSE_SWIGLU = 2, /* W_down (silu(W_gate h) * (W_up h)); ff_up holds the rows of gate and up INTERLEAVED (gate_0, up_0, gate_1, ...): [2 ff, width] */
+};
+enum ps_layer_form {
+    PS_LAYER_SEQUENTIAL = 0, /* x += norm_b(mixer(conv(norm1(x)))), then x += norm_b(ff(conv(norm2(x)))) */
+    PS_LAYER_PARALLEL   = 1, /* h = norm1(x); x += mixer(conv(h)) + ff(h): one norm, no norm behind the sublayers, only the mixer's input is filtered */
+};
+enum ps_rot_pairing { PS_ROT_HALVES = 0 /* (i, i + dims/2) */, PS_ROT_NEIGHBOURS = 1 /* (2i, 2i + 1) */ };
 
 /* Dense matrix [N rows = outputs][K = inputs], row-major, applied as W x.  host_bf16: N*K bfloat16 bit patterns.
  * as_f32 != 0 widens it to fp32 on the device (the fp32 compute mode). */
@@ -318,7 +330,7 @@ void ps_hip_dense_free(ps_hip_ctx *ctx, ps_dense *w);
 /* out[T][N] = alpha * (x[T][K] . W^T), device fp32 in and out (tests, micro-benchmarks; the model uses the same launchers) */
 int ps_hip_dense_matmul(ps_hip_ctx *ctx, const ps_dense *w, const float *x_dev, int T, float *out_dev, float alpha);
 
-typedef struct {
+typedef struct ps_seq_layer_s {
     int32_t kind;     /* ps_mixer_kind */
     int32_t heads, kv_heads, dim, vdim; /* q/k size per head, value size per head (wkv: vdim == dim) */
     int32_t conv_taps;                  /* delta: taps of the short convolutions on q / k / v */
@@ -341,6 +353,25 @@ typedef struct {
      * delta: conv [2*kv_heads*dim + heads*vdim][conv_taps] (rows q | k | v); a_log, dt_bias [heads]; onorm [vdim]
      * latent: qnorm [q_rank], kvnorm [kv_rank] */
     const float *mu, *decay0, *bonus, *onorm, *conv, *a_log, *dt_bias, *qnorm, *kvnorm;
+    /* ---- layer form and mixers side by side */
+    int32_t form;                       /* ps_layer_form */
+    float mix_scale;                    /* the mixer's output is multiplied by this (1 for a mixer on its own) */
+    const struct ps_seq_layer_s *beside; /* a second mixer that reads the same input; the layer's mixer output is the sum of both (each times its
+                                          * mix_scale).  Only its mixer fields are read.  NULL: none */
+    /* ---- windowed attention (PS_MIX_WINATTN); it also reads heads, kv_heads, dim, vdim, rot_dims (per head, the first rot_dims numbers turn),
+     * rot_base, window (0: everything before the token), scale, qnorm, out.
+     *   in_cat = rows of q | k | v | gate  ([heads*dim + kv_heads*dim + kv_heads*vdim + (gated ? heads : 0), width])
+     *   in_bias [rows of in_cat] or NULL; qnorm [heads*dim] / knorm [kv_heads*dim] plain weights of RMS norms over the WHOLE projection, or NULL: no norm;
+     *   temp [heads] multiplies a head's scores (NULL: 1); sink [heads] adds exp(sink) to a head's soft-max denominator (NULL: none) */
+    int32_t pool;                       /* tokens per pooled block behind the window (0: none) */
+    int32_t rot_pairing;                /* ps_rot_pairing */
+    int32_t gated;                      /* 1: a head's output is multiplied by sigmoid of its row of the gate projection */
+    float rot_factor;                   /* every rotary frequency is divided by this (linear position scaling; 0 is taken as 1) */
+    const float *in_bias, *knorm, *temp, *sink;
+    /* ---- gated linear attention (PS_MIX_GLA); it also reads heads, dim, vdim, decay_rank, onorm [vdim], out.
+     *   in_cat = rows of q | k | v | g | a1  ([2*heads*dim + 2*heads*vdim + decay_rank, width]); decay2 [heads*dim, decay_rank]; decay0 [heads*dim] its bias;
+     *   alpha = sigmoid(z)^(1/tau), q is scaled by dim^-1/2, the output is per-head RMS-normed (onorm shared by the heads) and multiplied by silu(g) */
+    float tau;
 } ps_seq_layer;
 
 typedef struct {
@@ -352,6 +383,11 @@ typedef struct {
     const ps_dense *embed, *head; /* [vocab, width] both */
     const float *final_norm;
     const ps_seq_layer *layers;
+    float embed_scale;   /* the embedding row is multiplied by this (0 is taken as 1) */
+    /* layers loop_start .. loop_stop - 1 run loop_times times in a row with the same weights, each pass with a state of its own; then the rest follow
+     * (loop_times <= 1: every layer runs once).  A "layer run" below is one execution of a layer. */
+    int32_t loop_start, loop_stop, loop_times;
+    int32_t max_context; /* most tokens a sequence may hold: sizes what grows with a sequence (the pooled blocks of PS_MIX_WINATTN); 0: 65536 */
 } ps_seq_desc;
 
 int ps_hip_seq_create(ps_hip_ctx *ctx, const ps_seq_desc *desc, ps_hip_seq **out);
@@ -371,8 +407,9 @@ int ps_hip_seq_forward(ps_hip_seq *m, int slot, const int32_t *tokens, int n, co
 /* Greedy single-token steps: feeds `token`, then its own arg-max, `steps` times (captured launch sequence, no host round trip
  * per token).  out_ids HOST int32[steps]. */
 int ps_hip_seq_decode_greedy(ps_hip_seq *m, int slot, int32_t token, int steps, int32_t *out_ids);
-/* diagnostics: with buf != NULL (device, [n_layers][max_batch][width] fp32) every forward of at most max_batch tokens leaves
- * the residual stream after each layer there */
+int ps_hip_seq_layer_runs(const ps_hip_seq *m); /* layer runs of one forward (the looped stretch counted every time) */
+/* diagnostics: with buf != NULL (device, [layer runs][max_batch][width] fp32) every forward of at most max_batch tokens leaves
+ * the residual stream after each layer run there */
 int ps_hip_seq_debug_layers(ps_hip_seq *m, float *buf_dev);
 /* bit 0: 1 = eager launches for the single-token step (default: hipGraph replay); bit 1: 1 = the unfused reference kernels
  * wherever a faster form exists (per-key attention, tiled mat-mul for single tokens) -- same results up to rounding */

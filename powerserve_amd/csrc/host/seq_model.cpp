@@ -127,6 +127,8 @@ void ranutar(const JsonValue &cfg, const SafeTensorsFile &st, SeqUploader &up, s
         const JsonValue &lc = ls[i], &mc = lc.at("mixer");
         const std::string p = "l" + std::to_string(i) + ".", m = p + "mix.", kind = lc.at("type").str;
         ps_seq_layer L{};
+        L.form = PS_LAYER_SEQUENTIAL;
+        L.mix_scale = 1.0f;
         L.norm1 = up.vec(st.f32(p + "norm1"));
         L.norm1b = up.vec(st.f32(p + "norm1b"));
         L.canon1 = up.vec(expect(st, p + "canon1", d.width, d.canon_taps));

@@ -34,6 +34,7 @@ struct dn_args {
     int act;
     float act_p, act_q, alpha;
     const float *mu, *shift0;
+    int accum;
 };
 
 // rows of A that exist and where they start (ring rows relative to the step's position)
@@ -67,6 +68,23 @@ static __device__ __forceinline__ float dn_epi(const dn_args &g, float acc, long
         acc = tanhf(acc);
     }
     return acc * g.alpha;
+}
+static __device__ __forceinline__ float dn_silu(float x) { return x / (1.f + expf(-x)); }
+// Result acc of (token t, weight row n) goes to its place.  other: the result of row n ^ 1 (the paired activation needs both; every lane of the wave calls
+// this with both values, only the even row stores).
+static __device__ __forceinline__ void dn_put(const dn_args &g, int t, long long n, float acc, float other, bool in) {
+    if (g.act == PSD_ACT_SILU_PAIR) {
+        if (in && !(n & 1)) {
+            float *p = g.out + (long long)t * g.ldo + (n >> 1);
+            const float v = dn_silu(acc) * other * g.alpha;
+            *p = g.accum ? *p + v : v;
+        }
+        return;
+    }
+    if (!in) return;
+    float *p = g.out + (long long)t * g.ldo + n;
+    const float v = dn_epi(g, acc, n);
+    *p = g.accum ? *p + v : v;
 }
 
 // ---------------------------------------------------------------------------------------------------- tiled mat-mul
@@ -161,7 +179,7 @@ __global__ __launch_bounds__(256) void dense_mm_kernel(dn_args g) {
             for (int e = 0; e < 4; e++) {
                 const int t = t0 + wm * 32 + i * 16 + lq * 4 + e;
                 const long long n = n0 + wn * 32 + j * 16 + lr;
-                if (t < T && n < g.N) g.out[(long long)t * g.ldo + n] = dn_epi(g, acc[i][j][e], n);
+                dn_put(g, t, n, acc[i][j][e], __shfl_xor(acc[i][j][e], 1, 64), t < T && n < g.N); // (row n ^ 1 is the neighbouring lane's)
             }
 }
 
@@ -243,11 +261,13 @@ __global__ __launch_bounds__(256) void dense_mv_kernel(dn_args g) {
         for (int r = 0; r < RW; r++)
 #pragma unroll
             for (int c = 0; c < C; c++) {
-                float v = acc[r][c];
 #pragma unroll
-                for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-                if (lane == 0 && nb + r < g.N && c < T) g.out[(long long)c * g.ldo + nb + r] = dn_epi(g, v, nb + r);
+                for (int o = 32; o > 0; o >>= 1) acc[r][c] += __shfl_xor(acc[r][c], o, 64);
             }
+#pragma unroll
+        for (int r = 0; r < RW; r++)
+#pragma unroll
+            for (int c = 0; c < C; c++) dn_put(g, c, nb + r, acc[r][c], acc[r ^ 1][c], lane == 0 && nb + r < g.N && c < T); // (nb is a multiple of four)
     }
 }
 
@@ -338,7 +358,7 @@ __global__ __launch_bounds__(256) void dense_mm_fast_kernel(dn_args g, const uns
             for (int e = 0; e < 4; e++) {
                 const int t = t0 + wm * 64 + i * 16 + lq * 4 + e;
                 const long long n = n0 + wn * 64 + j * 16 + lr;
-                if (t < T && n < g.N) g.out[(long long)t * g.ldo + n] = dn_epi(g, acc[i][j][e], n);
+                dn_put(g, t, n, acc[i][j][e], __shfl_xor(acc[i][j][e], 1, 64), t < T && n < g.N);
             }
 }
 
@@ -357,7 +377,7 @@ int psk_dense(hipStream_t st, const psk_dense_args &a) {
     dn_args g;
     g.w = a.w->data; g.a = a.a; g.lda = a.lda; g.a_row0 = a.a_row0; g.a_mod = a.a_mod; g.a_step = a.a_step; g.T = a.T;
     g.N = a.w->N; g.K = a.w->K; g.out = a.out; g.ldo = a.ldo; g.bias = a.bias; g.act = a.act; g.act_p = a.act_p; g.act_q = a.act_q;
-    g.alpha = a.alpha; g.mu = a.mu; g.shift0 = a.shift0;
+    g.alpha = a.alpha; g.mu = a.mu; g.shift0 = a.shift0; g.accum = a.accum;
     const bool bf = a.w->dtype == PS_BF16;
     const size_t kp4 = (size_t)((g.K + 7) / 8 * 8) * 4;
     if (!a.force_tiled && a.T <= 8) {
@@ -401,14 +421,15 @@ void psk_dense_widen(hipStream_t st, const uint16_t *bf16, int64_t n, float *out
     hipLaunchKernelGGL(dense_widen_kernel, dim3((unsigned)blocks), dim3(256), 0, st, bf16, (long long)n, out);
 }
 
-__global__ void dense_embed_kernel(const void *table, int is_bf16, long long K, const int32_t *tokens, const ps_seq_step *step, float *out, long long ldo) {
+__global__ void dense_embed_kernel(const void *table, int is_bf16, long long K, const int32_t *tokens, const ps_seq_step *step, float scale, float *out,
+                                   long long ldo) {
     const int t = blockIdx.x;
     const long long tok = (tokens ? tokens[t] : step->token0);
     for (long long k = threadIdx.x; k < K; k += blockDim.x)
-        out[t * ldo + k] = is_bf16 ? dn_bf2f(((const unsigned short *)table)[tok * K + k]) : ((const float *)table)[tok * K + k];
+        out[t * ldo + k] = (is_bf16 ? dn_bf2f(((const unsigned short *)table)[tok * K + k]) : ((const float *)table)[tok * K + k]) * scale;
 }
-void psk_embed(hipStream_t st, const ps_dense *table, const int32_t *tokens, const ps_seq_step *step, int T, float *out, int64_t ldo) {
-    hipLaunchKernelGGL(dense_embed_kernel, dim3(T), dim3(256), 0, st, table->data, table->dtype == PS_BF16 ? 1 : 0, (long long)table->K, tokens, step, out,
+void psk_embed(hipStream_t st, const ps_dense *table, const int32_t *tokens, const ps_seq_step *step, int T, float scale, float *out, int64_t ldo) {
+    hipLaunchKernelGGL(dense_embed_kernel, dim3(T), dim3(256), 0, st, table->data, table->dtype == PS_BF16 ? 1 : 0, (long long)table->K, tokens, step, scale, out,
                        (long long)ldo);
 }
 

@@ -4,6 +4,7 @@
 //   latent_prep_kernel   norms of the two latents, rotation of the shared key part, ring append
 //   latent_attn_kernel   one wave per (token, head) over per-head keys / values expanded from the ring rows of the window (the plain form)
 //   latent_attn_mfma_kernel / latent_absorbed_kernel (+ fold, combine, unfold): the matrix-core forms for a portion and for a single token, below
+#include "ps_attn_dev.h"
 #include "ps_seq.h"
 
 #include <cmath>
@@ -131,108 +132,6 @@ void psk_latent_attn(hipStream_t st, const ps_seq_step *step, int64_t ring_off, 
 // consecutive tokens of one head), and the single-token step in the ABSORBED form -- rows = heads, every head's query folded through its key
 // expansion into latent space (q~_h = W_uk,h^T q_h), keys AND values the ring's latents themselves, the value expansion applied afterwards to
 // the attended latent -- where the ring is read once for all heads and nothing is expanded per key.
-typedef float la_f4 __attribute__((ext_vector_type(4)));
-
-struct la_src { // where key j's row lives: base + ((j - sub) mod `mod`) * ld   (mod 0: no wrap)
-    const float *base;
-    long long ld, sub, mod;
-};
-static __device__ __forceinline__ const float *la_row(const la_src &s, long long j) {
-    long long r = j - s.sub;
-    if (s.mod > 0) r %= s.mod;
-    return s.base + r * s.ld;
-}
-
-// qs: this wave's 16 rows in LDS, row stride qld floats, [DK1 | DK2]; pt: its 16 x 17 patch.  rowpos(i): position of accumulator row i of this
-// lane (rows 4 (l / 16) + i), < 0 for a row that does not exist.  Keys j0 .. j0 + 15 are visible to a row at position p when j <= p, j > p - window
-// and j < jend.  NJ: accumulator tiles (DV <= 16 NJ).
-template <int NJ>
-static __device__ __forceinline__ void la_tile(const float *qs, int qld, float *pt, const la_src &k1, const la_src &k2, const la_src &vs, int DK1, int DK2, int DV,
-                                               long long j0, long long jend, const long long (&rowpos)[4], int window, float scale, float (&m)[4], float (&l)[4],
-                                               la_f4 (&acc)[NJ]) {
-    const int lane = threadIdx.x & 63, lr = lane & 15, lq = lane >> 4;
-    const long long jk = j0 + lr < jend ? j0 + lr : jend - 1; // (a key row that exists; masked below)
-    la_f4 s4 = {0.f, 0.f, 0.f, 0.f};
-    const float *kr1 = la_row(k1, jk) + 4 * lq, *kr2 = la_row(k2, jk) + 4 * lq, *qr = qs + lr * qld + 4 * lq;
-    // eight 16-byte key pieces in flight per lane ahead of their 32 matrix instructions
-    for (int g0 = 0; g0 < DK1 + DK2; g0 += 128) {
-        la_f4 b[8], a[8];
-#pragma unroll
-        for (int u = 0; u < 8; u++) {
-            const int g = g0 + 16 * u;
-            b[u] = g < DK1 ? *(const la_f4 *)(kr1 + g) : (g < DK1 + DK2 ? *(const la_f4 *)(kr2 + (g - DK1)) : la_f4{0.f, 0.f, 0.f, 0.f});
-        }
-#pragma unroll
-        for (int u = 0; u < 8; u++) {
-            const int g = g0 + 16 * u;
-            a[u] = g < DK1 + DK2 ? *(const la_f4 *)(qr + g) : la_f4{0.f, 0.f, 0.f, 0.f};
-        }
-#pragma unroll
-        for (int u = 0; u < 8; u++)
-            if (g0 + 16 * u < DK1 + DK2) {
-#pragma unroll
-                for (int e = 0; e < 4; e++) s4 = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u][e], b[u][e], s4, 0, 0, 0);
-            }
-    }
-    const long long j = j0 + lr;
-    float p[4], corr[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const bool vis = rowpos[i] >= 0 && j < jend && j <= rowpos[i] && j > rowpos[i] - window;
-        const float s = vis ? s4[i] * scale : -INFINITY;
-        float tm = s;
-#pragma unroll
-        for (int o = 1; o < 16; o <<= 1) tm = fmaxf(tm, __shfl_xor(tm, o, 64));
-        const float mn = fmaxf(m[i], tm);
-        corr[i] = mn == -INFINITY ? 1.f : expf(m[i] - mn);
-        p[i] = mn == -INFINITY ? 0.f : expf(s - mn);
-        float ts = p[i];
-#pragma unroll
-        for (int o = 1; o < 16; o <<= 1) ts += __shfl_xor(ts, o, 64);
-        l[i] = l[i] * corr[i] + ts;
-        m[i] = mn;
-    }
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int i = 0; i < 4; i++) pt[(4 * lq + i) * 17 + lr] = p[i];
-    __builtin_amdgcn_wave_barrier();
-    float pa[4];
-#pragma unroll
-    for (int s = 0; s < 4; s++) pa[s] = pt[lr * 17 + 4 * s + lq];
-    __builtin_amdgcn_wave_barrier();
-    const float *vr[4];
-#pragma unroll
-    for (int s = 0; s < 4; s++) {
-        const long long jv = j0 + 4 * s + lq < jend ? j0 + 4 * s + lq : jend - 1; // (weight 0 beyond the end)
-        vr[s] = la_row(vs, jv) + 4 * lr;
-    }
-    la_f4 bn[4];
-#pragma unroll
-    for (int s = 0; s < 4; s++) bn[s] = 4 * lr < DV ? *(const la_f4 *)(vr[s]) : la_f4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int J = 0; J < NJ / 4; J++) {
-        if (64 * J < DV) { // (uniform)
-            la_f4 b[4];
-#pragma unroll
-            for (int s = 0; s < 4; s++) b[s] = bn[s];
-            if (J + 1 < NJ / 4 && 64 * (J + 1) < DV) { // the next 64 columns' pieces are requested before this group's matrix instructions
-                const bool in = 64 * (J + 1) + 4 * lr < DV;
-#pragma unroll
-                for (int s = 0; s < 4; s++) bn[s] = in ? *(const la_f4 *)(vr[s] + 64 * (J + 1)) : la_f4{0.f, 0.f, 0.f, 0.f};
-            }
-#pragma unroll
-            for (int jj = 0; jj < 4; jj++) {
-                la_f4 a = acc[4 * J + jj];
-#pragma unroll
-                for (int i = 0; i < 4; i++) a[i] *= corr[i];
-#pragma unroll
-                for (int s = 0; s < 4; s++) a = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[s], b[s][jj], a, 0, 0, 0);
-                acc[4 * J + jj] = a;
-            }
-        }
-    }
-}
-
 // a prompt's portion: block = 64 consecutive tokens of one head (a wave per 16), keys / values expanded per head in kv (position first + row)
 // dynamic LDS: 4 x (16 x qld + 16 x 17)
 template <int NJ>
@@ -267,16 +166,22 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const ps_seq_step
     const la_src k1 = {kv + (long long)h * d, ldkv, first, 0};
     const la_src k2 = {step->state + ring_off + kv_rank, (long long)(kv_rank + dr), 0, cap};
     const la_src vs = {kv + (long long)H * d + (long long)h * dv, ldkv, first, 0};
-    long long rowpos[4];
+    long long rowlo[4], rowhi[4];
     float m[4], l[4];
     la_f4 acc[NJ];
 #pragma unroll
-    for (int i = 0; i < 4; i++) { rowpos[i] = t0 + 4 * lq + i < T ? pos0 + t0 + 4 * lq + i : -1; m[i] = -INFINITY; l[i] = 0.f; }
+    for (int i = 0; i < 4; i++) {
+        const long long rp = pos0 + t0 + 4 * lq + i;
+        const bool in = t0 + 4 * lq + i < T;
+        rowlo[i] = in && rp - window + 1 > 0 ? rp - window + 1 : 0;
+        rowhi[i] = in ? rp + 1 : 0;
+        m[i] = -INFINITY; l[i] = 0.f;
+    }
 #pragma unroll
     for (int j = 0; j < NJ; j++) acc[j] = la_f4{0.f, 0.f, 0.f, 0.f};
     const long long plast = pos0 + (t0 + 15 < T ? t0 + 15 : T - 1), pfirst = pos0 + t0;
     const long long lo = pfirst - window + 1 > 0 ? pfirst - window + 1 : 0;
-    for (long long j0 = lo; j0 <= plast; j0 += 16) la_tile<NJ>(qs, qld, pt, k1, k2, vs, d, dr, dv, j0, plast + 1, rowpos, window, scale, m, l, acc);
+    for (long long j0 = lo; j0 <= plast; j0 += 16) la_tile<NJ>(qs, qld, pt, k1, k2, vs, d, dr, dv, j0, plast + 1, rowlo, rowhi, scale, m, l, acc);
 #pragma unroll
     for (int J = 0; J < NJ / 4; J++)
 #pragma unroll
@@ -370,14 +275,14 @@ __global__ __launch_bounds__(256) void latent_absorbed_kernel(const ps_seq_step 
     const long long tile = (long long)blockIdx.x * 4 + wave, j0 = lo + tile * 16;
     const float *ring = step->state + ring_off;
     const la_src k1 = {ring, (long long)(R + dr), 0, cap}, k2 = {ring + R, (long long)(R + dr), 0, cap};
-    long long rowpos[4];
+    long long rowlo[4], rowhi[4];
     float m[4], l[4];
     la_f4 acc[NJ];
 #pragma unroll
-    for (int i = 0; i < 4; i++) { rowpos[i] = h0 + 4 * lq + i < H ? p : -1; m[i] = -INFINITY; l[i] = 0.f; }
+    for (int i = 0; i < 4; i++) { rowlo[i] = h0 + 4 * lq + i < H ? lo : 0; rowhi[i] = h0 + 4 * lq + i < H ? p + 1 : 0; m[i] = -INFINITY; l[i] = 0.f; }
 #pragma unroll
     for (int j = 0; j < NJ; j++) acc[j] = la_f4{0.f, 0.f, 0.f, 0.f};
-    if (j0 <= p) la_tile<NJ>(qs, qld, pt, k1, k2, k1, R, dr, R, j0, p + 1, rowpos, window, scale, m, l, acc);
+    if (j0 <= p) la_tile<NJ>(qs, qld, pt, k1, k2, k1, R, dr, R, j0, p + 1, rowlo, rowhi, scale, m, l, acc);
     // partial of (tile, head): [o[R], m, l, -, -] (rows of R + 4 floats: 16-byte stores)
 #pragma unroll
     for (int i = 0; i < 4; i++) {

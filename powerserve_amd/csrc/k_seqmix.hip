@@ -115,7 +115,7 @@ void psk_copy(hipStream_t st, const float *src, float *dst, int64_t n) {
 // A single token's sublayer boundary in one launch (one block):  x += y / rms(y) * (offset + wb)   (where y is given), then, where wn is given,
 // h = conv(x / rms(x) * (offset + wn)) with the convolution's residual form and its tail brought up to date -- three launches of the kernels above.
 __global__ __launch_bounds__(1024) void sq_boundary1_kernel(const ps_seq_step *step, float *x, const float *y, const float *wb, const float *wn, const float *cw,
-                                                            int taps, long long tail_off, float offset, float eps, long long n, float *h) {
+                                                            int taps, long long tail_off, float offset, float eps, long long n, float *h, float *hn) {
     __shared__ float red[16];
     const int tid = threadIdx.x, nw = blockDim.x >> 6;
     auto block_sum = [&](float v) {
@@ -146,6 +146,7 @@ __global__ __launch_bounds__(1024) void sq_boundary1_kernel(const ps_seq_step *s
     float *tail = step->state + tail_off;
     for (long long c = tid; c < n; c += blockDim.x) { // (a thread re-reads only what it wrote itself)
         const float v = x[c] * inv * (offset + wn[c]);
+        if (hn) hn[c] = v;
         float s = cw[c * taps + taps - 1] * v;
         for (int j = 0; j < taps - 1; j++) s = fmaf(cw[c * taps + j], tail[(long long)j * n + c], s);
         h[c] = v + s;
@@ -154,8 +155,8 @@ __global__ __launch_bounds__(1024) void sq_boundary1_kernel(const ps_seq_step *s
     }
 }
 void psk_boundary1(hipStream_t st, const ps_seq_step *step, float *x, const float *y, const float *wb, const float *wn, const float *cw, int taps, int64_t tail_off,
-                   float offset, float eps, int64_t n, float *h) {
-    hipLaunchKernelGGL(sq_boundary1_kernel, dim3(1), dim3(n >= 2048 ? 1024 : 256), 0, st, step, x, y, wb, wn, cw, taps, (long long)tail_off, offset, eps, (long long)n, h);
+                   float offset, float eps, int64_t n, float *h, float *hn) {
+    hipLaunchKernelGGL(sq_boundary1_kernel, dim3(1), dim3(n >= 2048 ? 1024 : 256), 0, st, step, x, y, wb, wn, cw, taps, (long long)tail_off, offset, eps, (long long)n, h, hn);
 }
 
 // ---------------------------------------------------------------------------------------------------- recurrent scans
@@ -185,22 +186,27 @@ static __device__ __forceinline__ float sq_col_sum(float v, int R) {
     return v;
 }
 
+// The scan of a state with a decay per key channel, S [d][dv] per head, in its two forms:
+//   GLA = 0 (wkv)  o_j = sum_i r_i (S_ij + bonus_i k_i v_j), then S_ij <- w_i S_ij + k_i v_j,  w = exp(-exp(z))
+//   GLA = 1        S_ij <- w_i S_ij + k_i v_j, then o_j = sum_i (qscale r_i) S_ij,              w = sigmoid(z)^inv_tau = exp(-softplus(-z) inv_tau)
 // LDS: rs, ks, ws [TC][dp] (dp = NR * R, rows >= d zero), sc [TC] (sum_i r_i bonus_i k_i)
-__global__ __launch_bounds__(256) void sq_wkv_scan_kernel(const ps_seq_step *step, long long state_off, const float *r, const float *k, const float *v, const float *z,
-                                                          long long ld, const float *bonus, int d, int R, int T, float *o, long long ldo) {
+template <int GLA>
+__global__ __launch_bounds__(256) void sq_decay_scan_kernel(const ps_seq_step *step, long long state_off, const float *r, const float *k, const float *v, const float *z,
+                                                            long long ld, long long ldz, const float *bonus, int d, int dv, float qscale, float inv_tau, int R, int T,
+                                                            float *o, long long ldo) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int dp = SQ_NR * R, cpb = 256 / R;
     float *rs = lds, *ks = rs + SQ_TC * dp, *ws = ks + SQ_TC * dp, *sc = ws + SQ_TC * dp;
     const int h = blockIdx.y, tid = threadIdx.x, s = tid % R, j = blockIdx.x * cpb + tid / R;
-    const bool col = j < d;
-    float *S0 = step->state + state_off + (long long)h * d * d;
+    const bool col = j < dv;
+    float *S0 = step->state + state_off + (long long)h * d * dv;
     float S[SQ_NR];
 #pragma unroll
     for (int m = 0; m < SQ_NR; m++) {
         const int i = s * SQ_NR + m;
-        S[m] = (col && i < d) ? S0[(long long)i * d + j] : 0.f;
+        S[m] = (col && i < d) ? S0[(long long)i * dv + j] : 0.f;
     }
-    const long long hb = (long long)h * d;
+    const long long hb = (long long)h * d, vb = (long long)h * dv;
     // the next round's inputs are requested before the current round's steps run, and land in LDS after them
     float pa[SQ_PF], pb[SQ_PF], pc[SQ_PF], pv[SQ_TC];
     auto fetch = [&](int t0) {
@@ -212,10 +218,10 @@ __global__ __launch_bounds__(256) void sq_wkv_scan_kernel(const ps_seq_step *ste
             const long long at = (long long)(t0 + (in ? t : 0)) * ld + hb + (in ? i : 0);
             pa[e] = in ? r[at] : 0.f;
             pb[e] = in ? k[at] : 0.f;
-            pc[e] = in ? z[at] : -INFINITY; // exp(-exp(-inf)) = 1: with k = 0 a token that is not there leaves the state alone
+            pc[e] = in ? z[(long long)(t0 + t) * ldz + hb + i] : (GLA ? INFINITY : -INFINITY); // w = 1: with k = 0 a token that is not there leaves the state alone
         }
 #pragma unroll
-        for (int t = 0; t < SQ_TC; t++) pv[t] = (col && t < nt) ? v[(long long)(t0 + t) * ld + hb + j] : 0.f;
+        for (int t = 0; t < SQ_TC; t++) pv[t] = (col && t < nt) ? v[(long long)(t0 + t) * ld + vb + j] : 0.f;
     };
     fetch(0);
     for (int t0 = 0; t0 < T; t0 += SQ_TC) {
@@ -225,9 +231,9 @@ __global__ __launch_bounds__(256) void sq_wkv_scan_kernel(const ps_seq_step *ste
         for (int e = 0; e < SQ_PF; e++) {
             const int x = tid + 256 * e;
             if (x < SQ_TC * dp) {
-                rs[x] = pa[e];
+                rs[x] = GLA ? pa[e] * qscale : pa[e];
                 ks[x] = pb[e];
-                ws[x] = expf(-expf(pc[e]));
+                ws[x] = GLA ? expf(-sq_softplus(-pc[e]) * inv_tau) : expf(-expf(pc[e]));
             }
         }
         float vj[SQ_TC];
@@ -235,7 +241,7 @@ __global__ __launch_bounds__(256) void sq_wkv_scan_kernel(const ps_seq_step *ste
         for (int t = 0; t < SQ_TC; t++) vj[t] = pv[t];
         __syncthreads();
         if (t0 + SQ_TC < T) fetch(t0 + SQ_TC);
-        for (int t = tid >> 6; t < SQ_TC; t += 4) { // one wave per token
+        for (int t = tid >> 6; !GLA && t < SQ_TC; t += 4) { // one wave per token
             float a = 0.f;
             for (int i = tid & 63; i < d; i += 64) a += rs[t * dp + i] * bonus[hb + i] * ks[t * dp + i];
 #pragma unroll
@@ -254,27 +260,39 @@ __global__ __launch_bounds__(256) void sq_wkv_scan_kernel(const ps_seq_step *ste
                     const sq_f4 r4 = rt[m4], k4 = kt[m4], w4 = wt[m4];
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
-                        pp[e] = fmaf(r4[e], S[4 * m4 + e], pp[e]);
-                        S[4 * m4 + e] = fmaf(w4[e], S[4 * m4 + e], k4[e] * vj[t]);
+                        if constexpr (GLA) {
+                            S[4 * m4 + e] = fmaf(w4[e], S[4 * m4 + e], k4[e] * vj[t]);
+                            pp[e] = fmaf(r4[e], S[4 * m4 + e], pp[e]);
+                        } else {
+                            pp[e] = fmaf(r4[e], S[4 * m4 + e], pp[e]);
+                            S[4 * m4 + e] = fmaf(w4[e], S[4 * m4 + e], k4[e] * vj[t]);
+                        }
                     }
                 }
                 const float p = sq_col_sum((pp[0] + pp[1]) + (pp[2] + pp[3]), R);
-                if (col && s == 0 && t < nt) o[(long long)(t0 + t) * ldo + hb + j] = fmaf(vj[t], sc[t], p);
+                if (col && s == 0 && t < nt) o[(long long)(t0 + t) * ldo + vb + j] = GLA ? p : fmaf(vj[t], sc[t], p);
             }
         }
     }
 #pragma unroll
     for (int m = 0; m < SQ_NR; m++) {
         const int i = s * SQ_NR + m;
-        if (col && i < d) S0[(long long)i * d + j] = S[m];
+        if (col && i < d) S0[(long long)i * dv + j] = S[m];
     }
 }
 void psk_wkv_scan(hipStream_t st, const ps_seq_step *step, int64_t state_off, const float *r, const float *k, const float *v, const float *z, int64_t ld,
                   const float *bonus, int H, int d, int T, float *o, int64_t ldo) {
     const int R = sq_lanes_per_col(d), cpb = 256 / R;
     const size_t lds = (size_t)(3 * SQ_TC * SQ_NR * R + SQ_TC) * 4;
-    hipLaunchKernelGGL(sq_wkv_scan_kernel, dim3((d + cpb - 1) / cpb, H), dim3(256), lds, st, step, (long long)state_off, r, k, v, z, (long long)ld, bonus, d, R, T, o,
-                       (long long)ldo);
+    hipLaunchKernelGGL(sq_decay_scan_kernel<0>, dim3((d + cpb - 1) / cpb, H), dim3(256), lds, st, step, (long long)state_off, r, k, v, z, (long long)ld, (long long)ld, bonus, d, d, 1.f, 1.f,
+                       R, T, o, (long long)ldo);
+}
+void psk_gla_scan(hipStream_t st, const ps_seq_step *step, int64_t state_off, const float *q, const float *k, const float *v, int64_t ld, const float *z, int64_t ldz,
+                  float tau, int H, int d, int dv, int T, float *o, int64_t ldo) {
+    const int R = sq_lanes_per_col(d), cpb = 256 / R;
+    const size_t lds = (size_t)(3 * SQ_TC * SQ_NR * R + SQ_TC) * 4;
+    hipLaunchKernelGGL(sq_decay_scan_kernel<1>, dim3((dv + cpb - 1) / cpb, H), dim3(256), lds, st, step, (long long)state_off, q, k, v, z, (long long)ld, (long long)ldz, nullptr, d, dv,
+                       1.f / sqrtf((float)d), 1.f / tau, R, T, o, (long long)ldo);
 }
 
 // LDS: qs, ks [TC][dp]; per token: g, beta, kq

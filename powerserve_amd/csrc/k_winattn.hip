@@ -1,0 +1,159 @@
+// Windowed attention with pooled blocks of the layer-list models (PS_MIX_WINATTN): grouped-query soft-max attention in which a token at
+// position p sees the `window` positions up to itself and, beside them, ONE key and value for every block of `pool` consecutive positions that
+// lies wholly before that window (the means of the block's keys / values as the ring holds them); a per-head sink adds exp(sink) to the
+// denominator, a per-head temperature multiplies the scores, a per-head sigmoid gate the output.  What a sequence keeps: a RING of the last
+// `cap` tokens' keys and values (row = position mod cap; cap >= window - 1 + the widest step) and the block means, one row per block, which
+// grow with the sequence.  Scores, soft-max and the weighted sums are fp32.
+//   winattn_prep_kernel    norms over the whole q / k projections, rotation, ring append            (one block per token)
+//   winattn_pool_kernel    block sums in position order, turned into means when a block is complete  (a thread per channel and block)
+//   winattn_kernel         one wave per (token, head) over [visible blocks | window]: the plain form, any size
+//   winattn_mfma_kernel    a portion on the fp32 matrix cores, 16 tokens of a head per wave (ps_attn_dev.h)
+//   winattn_step_kernel + winattn_merge_kernel   a single token: rows = the heads that share a key / value group, a key tile per wave
+#include "ps_attn_dev.h"
+#include "ps_seq.h"
+
+#include <cmath>
+
+static __device__ __forceinline__ float wa_wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+static __device__ __forceinline__ float wa_wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+// blocks of `pool` positions wholly before the window of a query at p: block b is seen when b pool + pool - 1 <= p - window
+static __device__ __forceinline__ long long wa_blocks(long long p, int window, int pool) {
+    const long long n = p - window + 1;
+    return (pool > 0 && n > 0) ? n / pool : 0;
+}
+
+// y[t] = [ q (H d) | k (G d) | v (G dv) | ... ].  q -> qo[t] normed and rotated; k (normed, rotated) and v -> ring row pos mod cap: [G d | G dv].
+__global__ __launch_bounds__(256) void winattn_prep_kernel(const ps_seq_step *step, long long ring_off, int cap, const float *y, long long ldy, const float *qnorm,
+                                                           const float *knorm, float eps, int H, int G, int d, int dv, int rot_dims, int pairing, const float *freq,
+                                                           float *qo, long long ldq) {
+    __shared__ float red[8];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const long long pos = step->pos0 + t;
+    const int nq = H * d, nk = G * d, nv = G * dv;
+    const float *qt = y + (long long)t * ldy, *kt = qt + nq, *vt = kt + nk;
+    float *ring = step->state + ring_off + (pos % cap) * (long long)(nk + nv);
+    float a = 0.f, b = 0.f;
+    if (qnorm) for (int i = tid; i < nq; i += 256) a += qt[i] * qt[i];
+    if (knorm) for (int i = tid; i < nk; i += 256) b += kt[i] * kt[i];
+    a = wa_wave_sum(a);
+    b = wa_wave_sum(b);
+    if ((tid & 63) == 0) { red[tid >> 6] = a; red[4 + (tid >> 6)] = b; }
+    __syncthreads();
+    const float ia = qnorm ? 1.f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)nq + eps) : 1.f;
+    const float ib = knorm ? 1.f / sqrtf((red[4] + red[5] + red[6] + red[7]) / (float)nk + eps) : 1.f;
+    const int half = rot_dims / 2;
+    // element i of a projection (c = its index in its head): normed, and where c < rot_dims turned together with its partner
+    auto turned = [&](const float *src, const float *w, float inv, int i) {
+        const int c = i % d;
+        const float self = src[i] * inv * (w ? w[i] : 1.f);
+        if (c >= 2 * half) return self;
+        int partner, pair;
+        bool first;
+        if (pairing == PS_ROT_NEIGHBOURS) { partner = i - c + (c ^ 1); pair = c >> 1; first = !(c & 1); }
+        else { first = c < half; partner = first ? i + half : i - half; pair = first ? c : c - half; }
+        const float other = src[partner] * inv * (w ? w[partner] : 1.f);
+        const float ang = (float)pos * freq[pair], cs = cosf(ang), sn = sinf(ang);
+        return first ? self * cs - other * sn : self * cs + other * sn;
+    };
+    for (int i = tid; i < nq; i += 256) qo[(long long)t * ldq + i] = turned(qt, qnorm, ia, i);
+    for (int i = tid; i < nk; i += 256) ring[i] = turned(kt, knorm, ib, i);
+    for (int i = tid; i < nv; i += 256) ring[nk + i] = vt[i];
+}
+
+// Block sums of the ring rows this step appended, in position order (so the result does not depend on how the tokens were cut into steps); a
+// block that the step completes is stored as its mean.  A block whose first position the step brings starts from zero: nothing is cleared.
+__global__ __launch_bounds__(256) void winattn_pool_kernel(const ps_seq_step *step, long long ring_off, int cap, long long pool_off, int pool, int rs) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= rs) return;
+    const long long pos0 = step->pos0, end = pos0 + step->n, b = pos0 / pool + blockIdx.y, pb = b * pool;
+    const long long from = pb > pos0 ? pb : pos0, to = pb + pool < end ? pb + pool : end;
+    if (from >= to) return;
+    const float *ring = step->state + ring_off;
+    float *mean = step->state + pool_off + b * rs;
+    float s = from == pb ? 0.f : mean[c];
+    for (long long p = from; p < to; p++) s += ring[(p % cap) * rs + c];
+    mean[c] = to == pb + pool ? s / (float)pool : s;
+}
+
+void psk_winattn_prep(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *y, int64_t ldy, const float *qnorm,
+                      const float *knorm, float eps, int H, int G, int d, int dv, int rot_dims, int pairing, const float *freq, int T, float *q, int64_t ldq) {
+    hipLaunchKernelGGL(winattn_prep_kernel, dim3(T), dim3(256), 0, st, step, (long long)ring_off, cap, y, (long long)ldy, qnorm, knorm, eps, H, G, d, dv, rot_dims, pairing,
+                       freq, q, (long long)ldq);
+    if (pool > 0) {
+        const int rs = G * (d + dv);
+        hipLaunchKernelGGL(winattn_pool_kernel, dim3((rs + 255) / 256, (T - 1) / pool + 2), dim3(256), 0, st, step, (long long)ring_off, cap, (long long)pool_off, pool, rs);
+    }
+}
+
+// the sink joins a finished online soft-max (m running maximum, l denominator): returns the factor for the accumulated values
+static __device__ __forceinline__ float wa_finish(float m, float l, const float *sink, int h) {
+    if (!sink) return 1.f / l;
+    const float sk = sink[h], M = fmaxf(m, sk), c = expf(m - M); // (m = -inf cannot happen: a token sees itself)
+    return c / (l * c + expf(sk - M));
+}
+static __device__ __forceinline__ float wa_sigmoid(float x) { return 1.f / (1.f + expf(-x)); }
+
+// dynamic LDS: qs [d], ps [64].  Keys in one index space: [visible blocks | window tokens].
+#define WA_NV 4 // value columns per lane: dv <= 256
+__global__ __launch_bounds__(64) void winattn_kernel(const ps_seq_step *step, long long ring_off, int cap, long long pool_off, int pool, const float *q, long long ldq,
+                                                     const float *gate, long long ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window,
+                                                     float scale, float *o, long long ldo) {
+    extern __shared__ float lds[];
+    float *qs = lds, *ps = lds + d;
+    const int t = blockIdx.x, h = blockIdx.y, g = h / (H / G), lane = threadIdx.x;
+    const long long p = step->pos0 + t, lo = p - window + 1 > 0 ? p - window + 1 : 0, nb = wa_blocks(p, window, pool), nkeys = nb + (p - lo + 1);
+    const float *qt = q + (long long)t * ldq + (long long)h * d;
+    for (int i = lane; i < d; i += 64) qs[i] = qt[i];
+    __syncthreads();
+    const long long rs = (long long)G * (d + dv);
+    const float *ring = step->state + ring_off, *means = step->state + pool_off;
+    auto row = [&](long long n) { return n < nb ? means + n * rs : ring + ((lo + n - nb) % cap) * rs; };
+    const float sc = scale * (temp ? temp[h] : 1.f);
+    float m = -INFINITY, l = 0.f, acc[WA_NV];
+#pragma unroll
+    for (int x = 0; x < WA_NV; x++) acc[x] = 0.f;
+    for (long long n0 = 0; n0 < nkeys; n0 += 64) {
+        const long long n = n0 + lane;
+        float s = -INFINITY;
+        if (n < nkeys) {
+            const float *kn = row(n) + (long long)g * d;
+            float a = 0.f;
+            for (int i = 0; i < d; i++) a = fmaf(qs[i], kn[i], a);
+            s = a * sc;
+        }
+        const float mn = fmaxf(m, wa_wave_max(s));
+        const float corr = expf(m - mn), pj = n < nkeys ? expf(s - mn) : 0.f;
+        l = l * corr + wa_wave_sum(pj);
+        m = mn;
+        __syncthreads();
+        ps[lane] = pj;
+        __syncthreads();
+        const int nk = (int)min((long long)64, nkeys - n0);
+#pragma unroll
+        for (int x = 0; x < WA_NV; x++) acc[x] *= corr;
+        for (int kk = 0; kk < nk; kk++) {
+            const float *vr = row(n0 + kk) + (long long)G * d + (long long)g * dv;
+            const float pk = ps[kk];
+#pragma unroll
+            for (int x = 0; x < WA_NV; x++)
+                if (lane + 64 * x < dv) acc[x] = fmaf(pk, vr[lane + 64 * x], acc[x]);
+        }
+    }
+    const float f = wa_finish(m, l, sink, h) * (gate ? wa_sigmoid(gate[(long long)t * ldg + h]) : 1.f);
+#pragma unroll
+    for (int x = 0; x < WA_NV; x++)
+        if (lane + 64 * x < dv) o[(long long)t * ldo + (long long)h * dv + lane + 64 * x] = acc[x] * f;
+}
+void psk_winattn(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *q, int64_t ldq, const float *gate,
+                 int64_t ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window, float scale, int T, float *o, int64_t ldo) {
+    hipLaunchKernelGGL(winattn_kernel, dim3(T, H), dim3(64), (size_t)(d + 64) * 4, st, step, (long long)ring_off, cap, (long long)pool_off, pool, q, (long long)ldq, gate,
+                       (long long)ldg, temp, sink, H, G, d, dv, window, scale, o, (long long)ldo);
+}

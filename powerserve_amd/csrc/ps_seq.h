@@ -20,7 +20,8 @@ struct ps_seq_step {
     int32_t _pad;
 };
 
-enum { PSD_ACT_NONE = 0, PSD_ACT_XIELU = 1, PSD_ACT_TANH = 2 };
+enum { PSD_ACT_NONE = 0, PSD_ACT_XIELU = 1, PSD_ACT_TANH = 2,
+       PSD_ACT_SILU_PAIR = 3 }; // rows 2i / 2i + 1 of W are a gate and its partner: out[t][i] = silu(row 2i) * (row 2i + 1), N / 2 outputs
 
 // out[t][n] = alpha * act(sum_k A(t, k) W[n][k] + bias[n]),  t < T
 //   A(t, k) = a[row(t)][k], row(t) = t, or (a_row0 + t) mod a_mod when a_mod > 0 (rows of a ring), or, where a_step is given, rows of the
@@ -38,6 +39,7 @@ struct psk_dense_args {
     const float *bias = nullptr;
     int act = PSD_ACT_NONE;
     float act_p = 0.f, act_q = 0.f, alpha = 1.f; // xIELU: act_p = softplus(p), act_q = 1/2 + softplus(q)
+    int accum = 0; // 1: out += the result (the residual stream takes a sublayer's output projection directly)
     const float *mu = nullptr, *shift0 = nullptr;
     int force_tiled = 0; // 1: the plain tiled mat-mul whatever the shape (A/B against the mat-vec and the wide mat-mul)
     void *pack = nullptr; // scratch for the wide mat-mul's bfloat16 copy of A (T rounded up to 128 rows of K); without it the plain tiled kernel runs
@@ -45,8 +47,8 @@ struct psk_dense_args {
 };
 int psk_dense(hipStream_t st, const psk_dense_args &a);
 void psk_dense_widen(hipStream_t st, const uint16_t *bf16, int64_t n, float *out);
-// out[t][:] = table[token(t)][:]; tokens device int32 (step != NULL and T == 1: the token is step->token0)
-void psk_embed(hipStream_t st, const ps_dense *table, const int32_t *tokens, const ps_seq_step *step, int T, float *out, int64_t ldo);
+// out[t][:] = table[token(t)][:] * scale; tokens device int32 (step != NULL and T == 1: the token is step->token0)
+void psk_embed(hipStream_t st, const ps_dense *table, const int32_t *tokens, const ps_seq_step *step, int T, float scale, float *out, int64_t ldo);
 // out[r] = index of the first maximum of x[r][0..n)
 void psk_argmax_rows(hipStream_t st, const float *x, int64_t n, int rows, int32_t *out);
 
@@ -60,9 +62,10 @@ void psk_norm_residual(hipStream_t st, float *x, const float *y, const float *w,
 // (a residual around the convolution), mode 1: f = silu(sum).  The tail is brought up to date behind it.
 void psk_causal_conv(hipStream_t st, const ps_seq_step *step, int64_t tail_off, const float *in, int64_t ldi, const float *w, int taps, int mode,
                      int64_t C, int T, float *out, int64_t ldo);
-// One token's sublayer boundary fused: x += norm_b(y) (y may be NULL), then h = conv(norm(x)) in the residual form with the tail update (wn may be NULL: stop after x)
+// One token's sublayer boundary fused: x += norm_b(y) (y may be NULL), then h = conv(norm(x)) in the residual form with the tail update (wn may be NULL: stop after x);
+// hn (may be NULL) also receives norm(x) itself, for a sublayer that reads the unfiltered input
 void psk_boundary1(hipStream_t st, const ps_seq_step *step, float *x, const float *y, const float *wb, const float *wn, const float *cw, int taps, int64_t tail_off,
-                   float offset, float eps, int64_t n, float *h);
+                   float offset, float eps, int64_t n, float *h, float *hn);
 // state row copy: (step->state + off)[0..n) = src[0..n)
 void psk_state_store(hipStream_t st, const ps_seq_step *step, int64_t off, const float *src, int64_t n);
 void psk_fill(hipStream_t st, float *p, float v, int64_t n);
@@ -72,6 +75,10 @@ void psk_copy(hipStream_t st, const float *src, float *dst, int64_t n);
 // step->state + state_off.  o[t][h][j] = sum_i r_i (S_ij + bonus_i k_i v_j), then S_ij = w_i S_ij + k_i v_j.
 void psk_wkv_scan(hipStream_t st, const ps_seq_step *step, int64_t state_off, const float *r, const float *k, const float *v, const float *z, int64_t ld,
                   const float *bonus, int H, int d, int T, float *o, int64_t ldo);
+// gated linear attention scan.  q, k [T][H*d], v [T][H*dv] (row stride ld), z [T][H*d] (row stride ldz) the decay's pre-activation; state [H][d][dv] fp32.
+// Per head: S <- diag(sigmoid(z)^(1/tau)) S + k v^T, then o = S^T (q d^-1/2).
+void psk_gla_scan(hipStream_t st, const ps_seq_step *step, int64_t state_off, const float *q, const float *k, const float *v, int64_t ld, const float *z, int64_t ldz,
+                  float tau, int H, int d, int dv, int T, float *o, int64_t ldo);
 // gated delta rule scan.  q, k: [T][KH*d] after convolution + silu (unit-normalised here, q also times d^-1/2), v [T][H*dv] (row stride ld), braw / araw [T][H] (row stride ldb);
 // per head: g = exp(-exp(a_log) softplus(araw + dt_bias)), beta = sigmoid(braw); S = g S; u = beta (v - S^T k); S += k u^T; o = S^T q.
 void psk_delta_scan(hipStream_t st, const ps_seq_step *step, int64_t state_off, const float *q, const float *k, const float *v, const float *braw,
@@ -98,3 +105,14 @@ bool psk_latent_absorbed_ok(int d, int dr, int dv, int R);
 size_t psk_latent_absorbed_scratch(int H, int R, int window);
 void psk_latent_absorbed(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, const float *q, int qstride, const ps_dense *ukv, const float *freq,
                          int H, int d, int dr, int rot_dims, int dv, int R, int window, float scale, float *scratch, float *o);
+
+// ---- k_winattn.hip
+// y[t] = [ q (H d) | k (G d) | v (G dv) | ... ]: RMS norms over the whole q / k projections (qnorm / knorm, NULL: none), rotation of the first rot_dims numbers of
+// every head at the token's position (pairing: ps_rot_pairing; angle of pair i: pos * freq[i]); q -> q[t], k and v -> the ring row pos mod cap ([G d | G dv], ring at
+// step->state + ring_off); then the block means ([block][G d | G dv] at step->state + pool_off, pool > 0) are brought up to date.
+void psk_winattn_prep(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *y, int64_t ldy, const float *qnorm,
+                      const float *knorm, float eps, int H, int G, int d, int dv, int rot_dims, int pairing, const float *freq, int T, float *q, int64_t ldq);
+// o[t][h] = gate(t, h) * soft-max attention of q[t][h] over the visible block means and the window's ring rows, scores times scale * temp[h], exp(sink[h]) in the
+// denominator; gate [T][..] raw (sigmoid here; column h, row stride ldg), temp / sink / gate may be NULL.
+void psk_winattn(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *q, int64_t ldq, const float *gate,
+                 int64_t ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window, float scale, int T, float *o, int64_t ldo);

@@ -1,33 +1,43 @@
 // Layer-list models (include/ps_hip.h, "layer-list models"): the model object, its pool of sequence states and the step function.
 //
-// A step takes the next n tokens of ONE sequence from the state earlier steps left in its slot.  The residual stream is fp32; every
-// layer is  x += norm_b(mixer(conv(norm(x))))  then, where it has a feed-forward,  x += norm_b(ff(conv(norm(x)))).  What a sequence
-// carries: per layer the tails of the two input convolutions, and per mixer kind a token-shift row + the wkv state, the short
-// convolutions' tail + the delta-rule state, or the ring of latents -- one fp32 block per slot, rings last, the rest zeroed when
+// A step takes the next n tokens of ONE sequence from the state earlier steps left in its slot.  The residual stream is fp32; a
+// layer is either SEQUENTIAL,  x += norm_b(mixer(conv(norm(x))))  then, where it has a feed-forward,  x += norm_b(ff(conv(norm(x)))),
+// or PARALLEL,  h = norm(x); x += mixer(conv(h)) + ff(h).  A layer's mixer may have a second one beside it that reads the same input
+// (their outputs are added, each times its scale), and a stretch of layers may run several times in a row with the same weights: the
+// unit that owns state is the layer RUN.  What a sequence carries: per run the tails of the input convolutions, and per mixer kind a
+// token-shift row + the wkv state, the short convolutions' tail + the delta-rule state, the gated-linear-attention state, the ring of
+// latents, or the ring of keys and values + the block means -- one fp32 block per slot, rings and means last, the rest zeroed when
 // the slot is handed out.
 #include "ps_seq.h"
 
 #include <cmath>
 #include <cstring>
 #include <map>
+#include <memory>
 #include <string>
 #include <vector>
 
 namespace {
-struct LayerPlan {
+struct LayerPlan { // one layer RUN (and, as `side`, the second mixer of one)
     ps_seq_layer d;
-    int64_t off_canon1 = 0, off_canon2 = 0, off_shift = 0, off_conv = 0, off_S = 0, off_ring = 0;
-    int cap = 0;          // latent: ring rows
-    float *freq = nullptr; // latent: rot_dim / 2 angular frequencies
+    int layer = 0; // index into the descriptor's layers (runs of a looped layer share it, and its weights)
+    int64_t off_canon1 = 0, off_canon2 = 0, off_shift = 0, off_conv = 0, off_S = 0, off_ring = 0, off_pool = 0;
+    int cap = 0;          // latent / windowed attention: ring rows
+    int64_t pool_rows = 0; // windowed attention: block means held
+    float *freq = nullptr; // rot_dims / 2 angular frequencies (shared by the runs of a layer)
     float act_p = 0.f, act_q = 0.f;
     int64_t ncat = 0, cqkv = 0;
+    std::shared_ptr<LayerPlan> side;
 };
 } // namespace
 
 struct ps_hip_seq {
     ps_hip_ctx *ctx = nullptr;
     ps_seq_desc d;
-    std::vector<LayerPlan> L;
+    std::vector<LayerPlan> L; // layer runs in execution order
+    int64_t max_context = 0;
+    bool needs_context = false; // some mixer's memory grows with the sequence: a sequence may hold at most max_context tokens
+    float embed_scale = 1.f;
     int64_t state_floats = 0, zero_floats = 0;
     std::vector<float *> slot_state;
     std::vector<int64_t> slot_pos; // -1: free
@@ -79,32 +89,34 @@ int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) 
     int64_t off = 0, n1 = 0, n2 = 0, n3 = 0, n4 = 0, nkv = 0, nq = 0;
     auto fail = [&](const std::string &msg) { ps_hip_seq_destroy(m); return seq_fail(c, "seq_create: " + msg); };
     auto shape = [](const ps_dense *w, int64_t N, int64_t K) { return w && w->N == N && w->K == K; };
-    m->L.resize(desc->n_layers);
-    m->weight_bytes = dense_bytes(desc->head);
-    for (int i = 0; i < desc->n_layers; i++) {
-        LayerPlan &P = m->L[i];
-        P.d = desc->layers[i];
-        const ps_seq_layer &l = P.d;
-        const std::string at = "layer " + std::to_string(i) + ": ";
-        if (!l.norm1 || !l.norm1b || !l.canon1 || !l.out) return fail(at + "norm / canon / out missing");
-        P.off_canon1 = off; off += (int64_t)(desc->canon_taps - 1) * W;
-        if (l.ff_kind != PS_FF_NONE) {
-            if (l.ff_kind != PS_FF_DENSE_XIELU) return fail(at + "unknown feed-forward kind");
-            if (!l.norm2 || !l.norm2b || !l.canon2 || !shape(l.ff_up, l.ff, W) || !shape(l.ff_down, W, l.ff)) return fail(at + "feed-forward tensors");
-            P.off_canon2 = off; off += (int64_t)(desc->canon_taps - 1) * W;
-            const double sp = log1p(exp((double)l.ff_act_p)), sq = log1p(exp((double)l.ff_act_q));
-            P.act_p = (float)sp; P.act_q = (float)(0.5 + sq);
-            n4 = std::max<int64_t>(n4, l.ff);
-            m->weight_bytes += dense_bytes(l.ff_up) + dense_bytes(l.ff_down);
+    m->max_context = desc->max_context > 0 ? desc->max_context : 65536;
+    m->embed_scale = desc->embed_scale != 0.f ? desc->embed_scale : 1.f;
+    std::vector<int> order; // layer index of every run
+    {
+        const bool loop = desc->loop_times > 1;
+        if (loop && (desc->loop_start < 0 || desc->loop_stop > desc->n_layers || desc->loop_start >= desc->loop_stop)) return fail("loop_start / loop_stop");
+        for (int i = 0; i < desc->n_layers; i++) {
+            if (loop && i == desc->loop_start) {
+                for (int r = 0; r < desc->loop_times; r++)
+                    for (int j = desc->loop_start; j < desc->loop_stop; j++) order.push_back(j);
+                i = desc->loop_stop - 1;
+            } else {
+                order.push_back(i);
+            }
         }
+    }
+    m->weight_bytes = dense_bytes(desc->head);
+    // a mixer's sizes, its tensors' shapes, its zeroed state and its scratch needs (rings and block means are placed afterwards)
+    auto plan_mixer = [&](LayerPlan &P, const std::string &at) -> std::string {
+        const ps_seq_layer &l = P.d;
         const int64_t H = l.heads, d = l.dim, dv = l.vdim;
-        if (H <= 0 || d <= 0) return fail(at + "heads / dim");
+        if (H <= 0 || d <= 0 || !l.out) return at + "heads / dim / out";
         if (l.kind == PS_MIX_WKV) {
             const int64_t Hd = H * d;
-            if (d > 256) return fail(at + "wkv: dim > 256 is not supported by the scan kernel");
+            if (d > 256) return at + "wkv: dim > 256 is not supported by the scan kernel";
             if (!shape(l.in_r, Hd, W) || !shape(l.in_k, Hd, W) || !shape(l.in_v, Hd, W) || !shape(l.in_g, Hd, W) || !shape(l.decay1, l.decay_rank, W) ||
                 !shape(l.decay2, Hd, l.decay_rank) || !shape(l.out, W, Hd) || !l.mu || !l.decay0 || !l.bonus || !l.onorm)
-                return fail(at + "wkv tensors");
+                return at + "wkv tensors";
             P.off_shift = off; off += W;
             P.off_S = off; off += Hd * d;
             n1 = std::max(n1, 5 * Hd);
@@ -112,11 +124,11 @@ int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) 
             n3 = std::max(n3, Hd);
             m->weight_bytes += dense_bytes(l.in_r) * 4 + dense_bytes(l.decay1) + dense_bytes(l.decay2) + dense_bytes(l.out);
         } else if (l.kind == PS_MIX_DELTA) {
-            if (d > 256) return fail(at + "delta: dim > 256 is not supported by the scan kernel");
-            if (l.kv_heads <= 0 || H % l.kv_heads || dv <= 0 || l.conv_taps < 1) return fail(at + "delta sizes");
+            if (d > 256) return at + "delta: dim > 256 is not supported by the scan kernel";
+            if (l.kv_heads <= 0 || H % l.kv_heads || dv <= 0 || l.conv_taps < 1) return at + "delta sizes";
             P.cqkv = 2 * (int64_t)l.kv_heads * d + H * dv;
             P.ncat = P.cqkv + H * dv + 2 * H;
-            if (!shape(l.in_cat, P.ncat, W) || !shape(l.out, W, H * dv) || !l.conv || !l.a_log || !l.dt_bias || !l.onorm) return fail(at + "delta tensors");
+            if (!shape(l.in_cat, P.ncat, W) || !shape(l.out, W, H * dv) || !l.conv || !l.a_log || !l.dt_bias || !l.onorm) return at + "delta tensors";
             P.off_conv = off; off += (int64_t)(l.conv_taps - 1) * P.cqkv;
             P.off_S = off; off += H * d * dv;
             n1 = std::max(n1, P.ncat);
@@ -125,11 +137,11 @@ int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) 
             m->weight_bytes += dense_bytes(l.in_cat) + dense_bytes(l.out);
         } else if (l.kind == PS_MIX_LATENT) {
             if (dv <= 0 || dv > 256 || l.q_rank <= 0 || l.kv_rank <= 0 || l.rot_dim < 0 || l.rot_dims < 0 || l.rot_dims > l.rot_dim || (l.rot_dims & 1) || l.window < 1)
-                return fail(at + "latent sizes (vdim <= 256, even rot_dims <= rot_dim)");
+                return at + "latent sizes (vdim <= 256, even rot_dims <= rot_dim)";
             P.ncat = (int64_t)l.q_rank + l.kv_rank + l.rot_dim;
             if (!shape(l.in_cat, P.ncat, W) || !shape(l.uq, H * (d + l.rot_dim), l.q_rank) || !shape(l.ukv, H * d + H * dv, l.kv_rank) || !shape(l.out, W, H * dv) ||
                 !l.qnorm || !l.kvnorm)
-                return fail(at + "latent tensors");
+                return at + "latent tensors";
             P.cap = (int)(l.window - 1 + B);
             n1 = std::max(n1, P.ncat);
             nq = std::max(nq, H * (d + l.rot_dim));
@@ -137,14 +149,85 @@ int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) 
             n3 = std::max(n3, H * dv);
             nkv = std::max(nkv, (int64_t)(l.window - 1 + B) * (H * d + H * dv));
             m->weight_bytes += dense_bytes(l.in_cat) + dense_bytes(l.uq) + dense_bytes(l.ukv) + dense_bytes(l.out);
+        } else if (l.kind == PS_MIX_WINATTN) {
+            const int64_t G = l.kv_heads;
+            if (G <= 0 || H % G || dv <= 0 || dv > 256 || l.rot_dims < 0 || l.rot_dims > d || (l.rot_dims & 1) || l.window < 0 || l.pool < 0)
+                return at + "windowed attention sizes (heads a multiple of kv_heads, vdim <= 256, even rot_dims <= dim)";
+            if (l.rot_pairing != PS_ROT_HALVES && l.rot_pairing != PS_ROT_NEIGHBOURS) return at + "rot_pairing";
+            P.ncat = H * d + G * d + G * dv + (l.gated ? H : 0);
+            if (!shape(l.in_cat, P.ncat, W) || !shape(l.out, W, H * dv)) return at + "windowed attention tensors";
+            if (l.pool > 0 || l.window <= 0 || l.window > m->max_context) m->needs_context = true;
+            const int64_t window = l.window > 0 ? std::min<int64_t>(l.window, m->max_context) : m->max_context;
+            P.d.window = (int32_t)window;
+            P.cap = (int)(window - 1 + B);
+            P.pool_rows = l.pool > 0 ? m->max_context / l.pool + 1 : 0;
+            n1 = std::max(n1, P.ncat);
+            n2 = std::max(n2, H * d);
+            n3 = std::max(n3, H * dv);
+            m->weight_bytes += dense_bytes(l.in_cat) + dense_bytes(l.out);
+        } else if (l.kind == PS_MIX_GLA) {
+            if (d > 256) return at + "gated linear attention: dim > 256 is not supported by the scan kernel";
+            if (dv <= 0 || l.decay_rank <= 0 || !(l.tau > 0.f)) return at + "gated linear attention sizes";
+            P.ncat = 2 * H * d + 2 * H * dv + l.decay_rank;
+            if (!shape(l.in_cat, P.ncat, W) || !shape(l.decay2, H * d, l.decay_rank) || !shape(l.out, W, H * dv) || !l.decay0 || !l.onorm)
+                return at + "gated linear attention tensors";
+            P.off_S = off; off += H * d * dv;
+            n1 = std::max(n1, P.ncat);
+            n2 = std::max(n2, H * d);
+            n3 = std::max(n3, H * dv);
+            m->weight_bytes += dense_bytes(l.in_cat) + dense_bytes(l.decay2) + dense_bytes(l.out);
         } else {
-            return fail(at + "unknown mixer kind");
+            return at + "unknown mixer kind";
+        }
+        return "";
+    };
+    m->L.resize(order.size());
+    for (size_t ri = 0; ri < order.size(); ri++) {
+        LayerPlan &P = m->L[ri];
+        P.layer = order[ri];
+        P.d = desc->layers[P.layer];
+        const ps_seq_layer &l = P.d;
+        const std::string at = "layer " + std::to_string(P.layer) + ": ";
+        if (l.form != PS_LAYER_SEQUENTIAL && l.form != PS_LAYER_PARALLEL) return fail(at + "unknown layer form");
+        if (!l.norm1 || (l.form == PS_LAYER_SEQUENTIAL && !l.norm1b) || !l.canon1) return fail(at + "norm / canon missing");
+        P.off_canon1 = off; off += (int64_t)(desc->canon_taps - 1) * W;
+        if (l.ff_kind != PS_FF_NONE) {
+            if (l.ff_kind != PS_FF_DENSE_XIELU && l.ff_kind != PS_FF_DENSE_SWIGLU) return fail(at + "unknown feed-forward kind");
+            const int64_t up_rows = l.ff_kind == PS_FF_DENSE_SWIGLU ? 2 * (int64_t)l.ff : l.ff;
+            if (!shape(l.ff_up, up_rows, W) || !shape(l.ff_down, W, l.ff)) return fail(at + "feed-forward tensors");
+            if (l.form == PS_LAYER_SEQUENTIAL) {
+                if (!l.norm2 || !l.norm2b || !l.canon2) return fail(at + "feed-forward norm / canon missing");
+                P.off_canon2 = off; off += (int64_t)(desc->canon_taps - 1) * W;
+            }
+            const double sp = log1p(exp((double)l.ff_act_p)), sq = log1p(exp((double)l.ff_act_q));
+            P.act_p = (float)sp; P.act_q = (float)(0.5 + sq);
+            n4 = std::max<int64_t>(n4, l.ff);
+            m->weight_bytes += dense_bytes(l.ff_up) + dense_bytes(l.ff_down);
+        }
+        std::string e = plan_mixer(P, at);
+        if (!e.empty()) return fail(e);
+        if (l.beside) {
+            P.side = std::make_shared<LayerPlan>();
+            P.side->layer = P.layer;
+            P.side->d = *l.beside;
+            if (P.side->d.beside) return fail(at + "a mixer beside another has none beside itself");
+            e = plan_mixer(*P.side, at + "second mixer: ");
+            if (!e.empty()) return fail(e);
         }
     }
     n2 = std::max(n2, m->n_t2q + nq);
     m->zero_floats = off;
-    for (auto &P : m->L)
+    auto mixers = [&](auto &&f) { // every mixer plan, second ones included
+        for (auto &P : m->L) { f(P); if (P.side) f(*P.side); }
+    };
+    mixers([&](LayerPlan &P) {
         if (P.d.kind == PS_MIX_LATENT) { off = (off + 3) / 4 * 4; P.off_ring = off; off += (int64_t)P.cap * (P.d.kv_rank + P.d.rot_dim); } // (16-byte rows for the matrix-core kernels)
+        if (P.d.kind == PS_MIX_WINATTN) {
+            const int64_t rs = (int64_t)P.d.kv_heads * (P.d.dim + P.d.vdim);
+            off = (off + 3) / 4 * 4; P.off_ring = off; off += (int64_t)P.cap * rs;
+            off = (off + 3) / 4 * 4; P.off_pool = off; off += P.pool_rows * rs;
+        }
+    });
     m->state_floats = off;
     auto alloc = [&](void **p, size_t bytes) {
         if (ps_dev_malloc(p, bytes + 256) != hipSuccess) return false;
@@ -152,14 +235,20 @@ int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) 
         return true;
     };
     bool ok = true;
-    for (auto &P : m->L)
-        if (P.d.kind == PS_MIX_LATENT && P.d.rot_dims > 0) {
-            const int half = P.d.rot_dims / 2;
-            std::vector<float> f(half);
-            for (int i = 0; i < half; i++) f[i] = (float)pow((double)P.d.rot_base, -2.0 * i / (double)P.d.rot_dims);
-            ok = ok && alloc((void **)&P.freq, half * 4);
-            if (ok) ok = hipMemcpyAsync(P.freq, f.data(), half * 4, hipMemcpyHostToDevice, c->stream) == hipSuccess && hipStreamSynchronize(c->stream) == hipSuccess;
-        }
+    std::map<const void *, float *> freq_of; // one table per layer (keyed by its output matrix), shared by its runs
+    mixers([&](LayerPlan &P) {
+        const bool lat = P.d.kind == PS_MIX_LATENT, win = P.d.kind == PS_MIX_WINATTN;
+        if (!(lat || win) || P.d.rot_dims <= 0 || !ok) return;
+        auto it = freq_of.find(P.d.out);
+        if (it != freq_of.end()) { P.freq = it->second; return; }
+        const int half = P.d.rot_dims / 2;
+        const double factor = win && P.d.rot_factor != 0.f ? (double)P.d.rot_factor : 1.0;
+        std::vector<float> f(half);
+        for (int i = 0; i < half; i++) f[i] = (float)(pow((double)P.d.rot_base, -2.0 * i / (double)P.d.rot_dims) / factor);
+        ok = ok && alloc((void **)&P.freq, half * 4);
+        if (ok) ok = hipMemcpyAsync(P.freq, f.data(), half * 4, hipMemcpyHostToDevice, c->stream) == hipSuccess && hipStreamSynchronize(c->stream) == hipSuccess;
+        freq_of[P.d.out] = P.freq;
+    });
     ok = ok && alloc((void **)&m->step, sizeof(ps_seq_step)) && alloc((void **)&m->x, B * W * 4) && alloc((void **)&m->hn, B * W * 4) && alloc((void **)&m->h, B * W * 4) &&
          alloc((void **)&m->y, B * W * 4) && alloc((void **)&m->t1, B * std::max<int64_t>(n1, 1) * 4) && alloc((void **)&m->t2, B * std::max<int64_t>(n2, 1) * 4) &&
          alloc((void **)&m->t3, B * std::max<int64_t>(n3, 1) * 4) && alloc((void **)&m->t4, B * std::max<int64_t>(n4, 1) * 4) &&
@@ -167,17 +256,18 @@ int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) 
          alloc((void **)&m->tokens, B * 4) && alloc((void **)&m->want, B * 4) && alloc((void **)&m->amax, B * 4);
     {
         size_t ab = 0;
-        for (auto &P : m->L)
+        mixers([&](LayerPlan &P) {
             if (P.d.kind == PS_MIX_LATENT && psk_latent_absorbed_ok(P.d.dim, P.d.rot_dim, P.d.vdim, P.d.kv_rank))
                 ab = std::max(ab, psk_latent_absorbed_scratch(P.d.heads, P.d.kv_rank, P.d.window));
+        });
         if (ab) ok = ok && alloc((void **)&m->abs_scratch, ab);
     }
     if (desc->compute == 0) { // the wide mat-mul's operand copy: the widest input of any matrix x a portion's rows, or the window's rows x the latent
         int64_t kmax = W, kvrows = 0, kvk = 0;
-        for (auto &P : m->L) {
+        mixers([&](LayerPlan &P) {
             kmax = std::max<int64_t>({kmax, P.d.ff, P.d.heads * (int64_t)std::max(P.d.dim, P.d.vdim), P.d.q_rank, P.d.decay_rank});
             if (P.d.kind == PS_MIX_LATENT) { kvrows = std::max<int64_t>(kvrows, P.d.window - 1 + B); kvk = std::max<int64_t>(kvk, P.d.kv_rank); }
-        }
+        });
         const int64_t r128 = (B + 127) / 128 * 128, kv128 = (kvrows + 127) / 128 * 128;
         m->pack_bytes = (size_t)std::max(r128 * kmax, kv128 * kvk) * 2;
         ok = ok && alloc(&m->pack, m->pack_bytes);
@@ -221,29 +311,30 @@ int ps_hip_seq_release(ps_hip_seq *m, int slot) {
 int64_t ps_hip_seq_position(const ps_hip_seq *m, int slot) { return (slot < 0 || slot >= (int)m->slot_pos.size()) ? -1 : m->slot_pos[slot]; }
 size_t ps_hip_seq_slot_bytes(const ps_hip_seq *m) { return (size_t)m->state_floats * 4; }
 uint64_t ps_hip_seq_weight_bytes_per_token(const ps_hip_seq *m) { return m->weight_bytes; }
+int ps_hip_seq_layer_runs(const ps_hip_seq *m) { return (int)m->L.size(); }
 int ps_hip_seq_debug_layers(ps_hip_seq *m, float *buf) { m->dbg_layers = buf; return 0; }
 int ps_hip_seq_set_mode(ps_hip_seq *m, int mode) { m->mode = mode; return 0; }
 
 } // extern "C"
 
 // The launches of one portion: T <= max_batch tokens (device ids in m->tokens, or the step's own token0 when from_step) of the slot whose state
-// pointer is `state`.  kv_rows_hint < 0: the step's position is known on the host (pos0); >= 0: a captured sequence that must hold for any
-// position -- the window's expansion is launched for its most rows and cut on the device.
+// pointer is `state`.  any_pos: a captured sequence that must hold for any position -- whatever depends on the position (the rows of a window's
+// expansion, the visible blocks) is launched for its most and cut on the device; otherwise the step's position is known on the host (pos0).
 static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool any_pos, bool from_step) {
     hipStream_t st = m->ctx->stream;
     const ps_seq_desc &D = m->d;
     const int64_t W = D.width;
     const bool tiled = (m->mode & 2) != 0;
-    psk_embed(st, D.embed, from_step ? nullptr : m->tokens, m->step, T, m->x, W);
+    psk_embed(st, D.embed, from_step ? nullptr : m->tokens, m->step, T, m->embed_scale, m->x, W);
     auto mm = [&](const ps_dense *w, const float *a, int64_t lda, float *out, int64_t ldo) {
         psk_dense_args g;
         g.w = w; g.a = a; g.lda = lda; g.T = T; g.out = out; g.ldo = ldo; g.force_tiled = tiled; g.pack = m->pack; g.pack_bytes = m->pack_bytes;
         return g;
     };
-    // a sublayer boundary: x += norm_b(y) (after a sublayer), then h = conv(norm(x)) (in front of the next one); one launch for a single token
+    // a sublayer boundary: x += norm_b(y) (after a sublayer), then hn = norm(x), h = conv(hn) (in front of the next one); one launch for a single token
     auto boundary = [&](const float *y, const float *wb, const float *wn, const float *cw, int64_t tail_off) {
         if (T == 1 && !tiled) {
-            psk_boundary1(st, m->step, m->x, y, wb, wn, cw, D.canon_taps, tail_off, D.norm_offset, D.norm_eps, W, m->h);
+            psk_boundary1(st, m->step, m->x, y, wb, wn, cw, D.canon_taps, tail_off, D.norm_offset, D.norm_eps, W, m->h, m->hn);
             return;
         }
         if (y) psk_norm_residual(st, m->x, y, wb, D.norm_offset, D.norm_eps, W, T);
@@ -252,12 +343,15 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
             psk_causal_conv(st, m->step, tail_off, m->hn, W, cw, D.canon_taps, 0, W, T, m->h, W);
         }
     };
-    boundary(nullptr, nullptr, m->L[0].d.norm1, m->L[0].d.canon1, m->L[0].off_canon1);
-    for (int li = 0; li < D.n_layers; li++) {
-        const LayerPlan &P = m->L[li];
+    // One mixer on the input m->h.  Its output projection writes m->y (into == NULL) or adds out_scale times its result to `into`.
+    auto mixer = [&](const LayerPlan &P, float *into, float out_scale) {
         const ps_seq_layer &l = P.d;
         const int64_t H = l.heads, d = l.dim, dv = l.vdim;
-        const LayerPlan *next = li + 1 < D.n_layers ? &m->L[li + 1] : nullptr;
+        auto out_proj = [&](const float *a, int64_t lda) {
+            auto g = mm(l.out, a, lda, into ? into : m->y, W);
+            g.alpha = out_scale; g.accum = into ? 1 : 0;
+            psk_dense(st, g);
+        };
         if (l.kind == PS_MIX_WKV) {
             const int64_t Hd = H * d, NW = 5 * Hd;
             const ps_dense *ws[4] = {l.in_r, l.in_k, l.in_v, l.in_g};
@@ -277,7 +371,7 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
             psk_state_store(st, m->step, P.off_shift, m->h + (int64_t)(T - 1) * W, W);
             psk_wkv_scan(st, m->step, P.off_S, m->t1, m->t1 + Hd, m->t1 + 2 * Hd, m->t1 + 4 * Hd, NW, l.bonus, (int)H, (int)d, T, m->t3, Hd);
             psk_headnorm_gate(st, m->t3, Hd, m->t1 + 3 * Hd, NW, l.onorm, (int)d, D.norm_eps, (int)H, (int)d, T);
-            psk_dense(st, mm(l.out, m->t3, Hd, m->y, W));
+            out_proj(m->t3, Hd);
         } else if (l.kind == PS_MIX_DELTA) {
             const int64_t KHd = (int64_t)l.kv_heads * d, Hv = H * dv;
             psk_dense(st, mm(l.in_cat, m->h, W, m->t1, P.ncat));
@@ -285,7 +379,29 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
             psk_delta_scan(st, m->step, P.off_S, m->t2, m->t2 + KHd, m->t2 + 2 * KHd, m->t1 + P.cqkv + Hv, m->t1 + P.cqkv + Hv + H, P.cqkv, P.ncat, l.a_log, l.dt_bias,
                            (int)H, l.kv_heads, (int)d, (int)dv, T, m->t3, Hv);
             psk_headnorm_gate(st, m->t3, Hv, m->t1 + P.cqkv, P.ncat, l.onorm, 0, D.norm_eps, (int)H, (int)dv, T);
-            psk_dense(st, mm(l.out, m->t3, Hv, m->y, W));
+            out_proj(m->t3, Hv);
+        } else if (l.kind == PS_MIX_GLA) {
+            // t1 = [ q | k | v | g | a1 ]; the decay's second matrix (with its bias) -> t2; scan -> t3; per-head norm and gate; out
+            const int64_t Hd = H * d, Hv = H * dv;
+            psk_dense(st, mm(l.in_cat, m->h, W, m->t1, P.ncat));
+            auto g2 = mm(l.decay2, m->t1 + 2 * Hd + 2 * Hv, P.ncat, m->t2, Hd);
+            g2.bias = l.decay0;
+            psk_dense(st, g2);
+            psk_gla_scan(st, m->step, P.off_S, m->t1, m->t1 + Hd, m->t1 + 2 * Hd, P.ncat, m->t2, Hd, l.tau, (int)H, (int)d, (int)dv, T, m->t3, Hv);
+            psk_headnorm_gate(st, m->t3, Hv, m->t1 + 2 * Hd + Hv, P.ncat, l.onorm, 0, D.norm_eps, (int)H, (int)dv, T);
+            out_proj(m->t3, Hv);
+        } else if (l.kind == PS_MIX_WINATTN) {
+            // t1 = [ q | k | v | gate ] (+ bias); norms, rotation, ring append and block means; attention -> t3; out
+            const int64_t G = l.kv_heads, Hd = H * d, Hv = H * dv;
+            auto g = mm(l.in_cat, m->h, W, m->t1, P.ncat);
+            g.bias = l.in_bias;
+            psk_dense(st, g);
+            psk_winattn_prep(st, m->step, P.off_ring, P.cap, P.off_pool, l.pool, m->t1, P.ncat, l.qnorm, l.knorm, D.norm_eps, (int)H, (int)G, (int)d, (int)dv, l.rot_dims,
+                             l.rot_pairing, P.freq, T, m->t2, Hd);
+            const float *gate = l.gated ? m->t1 + Hd + G * d + G * dv : nullptr;
+            psk_winattn(st, m->step, P.off_ring, P.cap, P.off_pool, l.pool, m->t2, Hd, gate, P.ncat, l.temp, l.sink, (int)H, (int)G, (int)d, (int)dv, l.window, l.scale, T,
+                        m->t3, Hv);
+            out_proj(m->t3, Hv);
         } else {
             const int64_t dr = l.rot_dim, rs = l.kv_rank + dr, Hv = H * dv, nq = H * (d + dr);
             float *cq = m->t2, *q = m->t2 + (int64_t)D.max_batch * m->n_t2q;
@@ -309,19 +425,49 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
                     psk_latent_attn(st, m->step, P.off_ring, P.cap, q, nq, m->kvx, H * d + Hv, P.freq, (int)H, (int)d, (int)dr, l.rot_dims, (int)dv, l.kv_rank, l.window,
                                     l.scale, T, m->t3, Hv);
             }
-            psk_dense(st, mm(l.out, m->t3, Hv, m->y, W));
+            out_proj(m->t3, Hv);
         }
-        const float *nn = next ? next->d.norm1 : nullptr, *nc = next ? next->d.canon1 : nullptr;
-        const int64_t no = next ? next->off_canon1 : 0;
-        if (l.ff_kind == PS_FF_DENSE_XIELU) {
-            boundary(m->y, l.norm1b, l.norm2, l.canon2, P.off_canon2);
-            auto g = mm(l.ff_up, m->h, W, m->t4, l.ff);
-            g.act = PSD_ACT_XIELU; g.act_p = P.act_p; g.act_q = P.act_q;
-            psk_dense(st, g);
-            psk_dense(st, mm(l.ff_down, m->t4, l.ff, m->y, W));
-            boundary(m->y, l.norm2b, nn, nc, no);
+    };
+    auto ff_up = [&](const LayerPlan &P, const float *in) {
+        const ps_seq_layer &l = P.d;
+        auto g = mm(l.ff_up, in, W, m->t4, l.ff);
+        if (l.ff_kind == PS_FF_DENSE_SWIGLU) g.act = PSD_ACT_SILU_PAIR;
+        else { g.act = PSD_ACT_XIELU; g.act_p = P.act_p; g.act_q = P.act_q; }
+        psk_dense(st, g);
+    };
+    const int n_runs = (int)m->L.size();
+    if (m->L[0].d.form == PS_LAYER_SEQUENTIAL) boundary(nullptr, nullptr, m->L[0].d.norm1, m->L[0].d.canon1, m->L[0].off_canon1);
+    for (int li = 0; li < n_runs; li++) {
+        const LayerPlan &P = m->L[li];
+        const ps_seq_layer &l = P.d;
+        const LayerPlan *next = li + 1 < n_runs ? &m->L[li + 1] : nullptr;
+        if (l.form == PS_LAYER_PARALLEL) {
+            // hn = norm(x), h = conv(hn); both mixers and the feed-forward add their output projections straight into the residual stream
+            boundary(nullptr, nullptr, l.norm1, l.canon1, P.off_canon1);
+            mixer(P, m->x, l.mix_scale);
+            if (P.side) mixer(*P.side, m->x, P.side->d.mix_scale);
+            if (l.ff_kind != PS_FF_NONE) {
+                ff_up(P, m->hn);
+                auto g = mm(l.ff_down, m->t4, l.ff, m->x, W);
+                g.accum = 1;
+                psk_dense(st, g);
+            }
         } else {
-            boundary(m->y, l.norm1b, nn, nc, no);
+            const bool summed = P.side != nullptr || l.mix_scale != 1.f;
+            if (summed) psk_fill(st, m->y, 0.f, (int64_t)T * W);
+            mixer(P, summed ? m->y : nullptr, l.mix_scale);
+            if (P.side) mixer(*P.side, m->y, P.side->d.mix_scale);
+            const bool nseq = next && next->d.form == PS_LAYER_SEQUENTIAL;
+            const float *nn = nseq ? next->d.norm1 : nullptr, *nc = nseq ? next->d.canon1 : nullptr;
+            const int64_t no = nseq ? next->off_canon1 : 0;
+            if (l.ff_kind != PS_FF_NONE) {
+                boundary(m->y, l.norm1b, l.norm2, l.canon2, P.off_canon2);
+                ff_up(P, m->h);
+                psk_dense(st, mm(l.ff_down, m->t4, l.ff, m->y, W));
+                boundary(m->y, l.norm2b, nn, nc, no);
+            } else {
+                boundary(m->y, l.norm1b, nn, nc, no);
+            }
         }
         if (m->dbg_layers && !any_pos) psk_copy(st, m->x, m->dbg_layers + (int64_t)li * D.max_batch * W, (int64_t)T * W);
     }
@@ -344,6 +490,7 @@ int ps_hip_seq_forward(ps_hip_seq *m, int slot, const int32_t *tokens, int n, co
     ps_hip_ctx *c = m->ctx;
     if (slot < 0 || slot >= (int)m->slot_pos.size() || m->slot_pos[slot] < 0) return seq_fail(c, "seq_forward: not a live slot");
     if (n <= 0 || !tokens) return seq_fail(c, "seq_forward: no tokens");
+    if (m->needs_context && m->slot_pos[slot] + n > m->max_context) return seq_fail(c, "seq_forward: the sequence would exceed max_context");
     for (int i = 0; i < n; i++)
         if (tokens[i] < 0 || tokens[i] >= m->d.vocab) return seq_fail(c, "seq_forward: token id outside the vocabulary");
     for (int i = 0; i < n_want; i++)
@@ -379,6 +526,7 @@ int ps_hip_seq_decode_greedy(ps_hip_seq *m, int slot, int32_t token, int steps, 
     if (slot < 0 || slot >= (int)m->slot_pos.size() || m->slot_pos[slot] < 0) return seq_fail(c, "seq_decode_greedy: not a live slot");
     if (steps <= 0) return 0;
     if (token < 0 || token >= m->d.vocab) return seq_fail(c, "seq_decode_greedy: token id outside the vocabulary");
+    if (m->needs_context && m->slot_pos[slot] + steps > m->max_context) return seq_fail(c, "seq_decode_greedy: the sequence would exceed max_context");
     PS_CHECK(c, hipSetDevice(c->device));
     if (steps > m->ids_cap) {
         if (m->ids) { PS_CHECK(c, hipStreamSynchronize(c->stream)); (void)ps_dev_free(m->ids); m->ids = nullptr; }
@@ -425,10 +573,14 @@ int ps_hip_seq_bench_kernel(ps_hip_seq *m, int which, int T, int reps, double *u
     PS_CHECK(c, hipSetDevice(c->device));
     std::vector<psk_dense_args> launches; // one per layer that has the matrix: every launch streams its own (cold) weights, as in a step
     for (const LayerPlan &P : m->L) {
-        if (P.d.ff_kind != PS_FF_DENSE_XIELU) continue;
+        if (P.d.ff_kind == PS_FF_NONE) continue;
         psk_dense_args g;
         g.T = T; g.pack = m->pack; g.pack_bytes = m->pack_bytes;
-        if (which == 0) { g.w = P.d.ff_up; g.a = m->h; g.lda = m->d.width; g.out = m->t4; g.ldo = P.d.ff; g.act = PSD_ACT_XIELU; g.act_p = P.act_p; g.act_q = P.act_q; }
+        if (which == 0) {
+            g.w = P.d.ff_up; g.a = m->h; g.lda = m->d.width; g.out = m->t4; g.ldo = P.d.ff;
+            if (P.d.ff_kind == PS_FF_DENSE_SWIGLU) g.act = PSD_ACT_SILU_PAIR;
+            else { g.act = PSD_ACT_XIELU; g.act_p = P.act_p; g.act_q = P.act_q; }
+        }
         else { g.w = P.d.ff_down; g.a = m->t4; g.lda = P.d.ff; g.out = m->y; g.ldo = m->d.width; }
         launches.push_back(g);
     }

@@ -35,7 +35,7 @@ EXPORTS = [
     "ps_hip_model_v_cache", "ps_hip_model_weight_bytes_per_token", "ps_hip_model_set_mode", "ps_hip_model_bench_gemv", "ps_hip_model_bench_matmul", "ps_hip_debug_timeline", "ps_hip_last_matmul_kernel", "ps_hip_debug_set", "ps_hip_debug_f16_gemm", "ps_hip_model_forward_tree", "ps_hip_model_prefill", "ps_hip_model_forward_lowered", "ps_hip_model_sync_check", "ps_hip_model_kv_mask",
     "ps_hip_soft_max", "ps_hip_model_kv_copy", "ps_hip_model_kv_save_tokens", "ps_hip_model_kv_unmask_tokens", "ps_hip_model_kv_append_tokens", "ps_hip_model_argmax",
     "ps_hip_dense_upload", "ps_hip_dense_free", "ps_hip_dense_matmul", "ps_hip_seq_create", "ps_hip_seq_destroy", "ps_hip_seq_acquire", "ps_hip_seq_release",
-    "ps_hip_seq_position", "ps_hip_seq_slot_bytes", "ps_hip_seq_forward", "ps_hip_seq_decode_greedy", "ps_hip_seq_debug_layers", "ps_hip_seq_set_mode",
+    "ps_hip_seq_position", "ps_hip_seq_slot_bytes", "ps_hip_seq_layer_runs", "ps_hip_seq_forward", "ps_hip_seq_decode_greedy", "ps_hip_seq_debug_layers", "ps_hip_seq_set_mode",
     "ps_hip_seq_weight_bytes_per_token", "ps_hip_seq_bench_kernel",
 ]
 # the part of EXPORTS that lib/libps_hip_seq.so has (everything else belongs to the quantized path)
@@ -87,18 +87,24 @@ def make_config(d: dict) -> LLMConfig:
 
 class SeqLayer(C.Structure):
     """ps_seq_layer (include/ps_hip.h)"""
-    _fields_ = ([(n, C.c_int32) for n in ("kind", "heads", "kv_heads", "dim", "vdim", "conv_taps", "decay_rank", "q_rank", "kv_rank", "rot_dim", "rot_dims", "window")] +
+
+
+SeqLayer._fields_ = ([(n, C.c_int32) for n in ("kind", "heads", "kv_heads", "dim", "vdim", "conv_taps", "decay_rank", "q_rank", "kv_rank", "rot_dim", "rot_dims", "window")] +
                 [("rot_base", C.c_float), ("scale", C.c_float), ("ff_kind", C.c_int32), ("ff", C.c_int32), ("ff_act_p", C.c_float), ("ff_act_q", C.c_float)] +
                 [(n, C.c_void_p) for n in ("norm1", "norm2", "norm1b", "norm2b", "canon1", "canon2")] +
                 [(n, C.c_void_p) for n in ("in_r", "in_k", "in_v", "in_g", "decay1", "decay2", "in_cat", "uq", "ukv", "out", "ff_up", "ff_down")] +
-                [(n, C.c_void_p) for n in ("mu", "decay0", "bonus", "onorm", "conv", "a_log", "dt_bias", "qnorm", "kvnorm")])
+                [(n, C.c_void_p) for n in ("mu", "decay0", "bonus", "onorm", "conv", "a_log", "dt_bias", "qnorm", "kvnorm")] +
+                [("form", C.c_int32), ("mix_scale", C.c_float), ("beside", C.POINTER(SeqLayer))] +
+                [("pool", C.c_int32), ("rot_pairing", C.c_int32), ("gated", C.c_int32), ("rot_factor", C.c_float)] +
+                [(n, C.c_void_p) for n in ("in_bias", "knorm", "temp", "sink")] + [("tau", C.c_float)])
 
 
 class SeqDesc(C.Structure):
     """ps_seq_desc (include/ps_hip.h)"""
     _fields_ = ([(n, C.c_int32) for n in ("n_layers", "width", "vocab", "canon_taps", "max_batch", "n_slots", "compute")] +
                 [("norm_eps", C.c_float), ("norm_offset", C.c_float), ("logit_scale", C.c_float)] +
-                [("embed", C.c_void_p), ("head", C.c_void_p), ("final_norm", C.c_void_p), ("layers", C.POINTER(SeqLayer))])
+                [("embed", C.c_void_p), ("head", C.c_void_p), ("final_norm", C.c_void_p), ("layers", C.POINTER(SeqLayer))] +
+                [("embed_scale", C.c_float)] + [(n, C.c_int32) for n in ("loop_start", "loop_stop", "loop_times", "max_context")])
 
 
 _LIB = None
@@ -157,7 +163,7 @@ def lib(seq_only_ok: bool = False) -> C.CDLL:
         "ps_hip_dense_matmul": (i32, [vp, vp, vp, i32, vp, C.c_float]),
         "ps_hip_seq_create": (i32, [vp, C.POINTER(SeqDesc), C.POINTER(vp)]), "ps_hip_seq_destroy": (None, [vp]),
         "ps_hip_seq_acquire": (i32, [vp, C.POINTER(i32)]), "ps_hip_seq_release": (i32, [vp, i32]), "ps_hip_seq_position": (i64, [vp, i32]),
-        "ps_hip_seq_slot_bytes": (sz, [vp]), "ps_hip_seq_forward": (i32, [vp, i32, vp, i32, vp, i32, vp, vp]),
+        "ps_hip_seq_slot_bytes": (sz, [vp]), "ps_hip_seq_layer_runs": (i32, [vp]), "ps_hip_seq_forward": (i32, [vp, i32, vp, i32, vp, i32, vp, vp]),
         "ps_hip_seq_decode_greedy": (i32, [vp, i32, i32, i32, vp]), "ps_hip_seq_debug_layers": (i32, [vp, vp]), "ps_hip_seq_set_mode": (i32, [vp, i32]),
         "ps_hip_seq_weight_bytes_per_token": (C.c_uint64, [vp]),
         "ps_hip_seq_bench_kernel": (i32, [vp, i32, i32, i32, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_double)]),

@@ -8,6 +8,14 @@ Ranutar: a list of layers, each  x += norm_b(mixer(conv(norm(x))))  and, where i
   delta             gated delta rule with short convolutions on q / k / v
   latent_attention  attention over a low-rank latent + one shared rotated key part, sliding window
 the norms RMS norms whose stored weight is the deviation from one, the feed-forward two dense matrices around the xIELU activation.
+
+Vobisun: PARALLEL layers,  h = norm(x); x += mixer(h + conv(h)) + ff(h), plain norm weights, a scaled embedding, a SiLU-gated feed-forward, a stretch
+of layers that runs several times with the same weights (config 'loop'; every pass has its own state), and the mixer type
+  parallel          two mixers side by side on the same input, their outputs added with a scale each:
+                    left  = grouped-query attention over a sliding window plus one mean key / value per block of 'pool' tokens wholly before the window,
+                            a sink in the soft-max denominator, a temperature per head, RMS norms over the whole q / k projections, rotary on neighbouring
+                            pairs of the first rot.dims numbers of a head with linearly scaled positions, a sigmoid gate per head;
+                    right = gated linear attention (a decay per key channel from a two-matrix projection).
 """
 from __future__ import annotations
 
@@ -20,8 +28,10 @@ import numpy as np
 from . import hip
 from .safetensors_io import SafeTensors
 
-MIX_WKV, MIX_DELTA, MIX_LATENT = 1, 2, 3
-FF_NONE, FF_DENSE_XIELU = 0, 1
+MIX_WKV, MIX_DELTA, MIX_LATENT, MIX_WINATTN, MIX_GLA = 1, 2, 3, 4, 5
+FF_NONE, FF_DENSE_XIELU, FF_DENSE_SWIGLU = 0, 1, 2
+LAYER_SEQUENTIAL, LAYER_PARALLEL = 0, 1
+ROT_HALVES, ROT_NEIGHBOURS = 0, 1
 
 
 class ConfigError(ValueError):
@@ -77,6 +87,7 @@ def _ranutar_layers(cfg: dict, st: SafeTensors, up) -> tuple[list, dict]:
             L.qnorm, L.kvnorm = up.vec(st.f32(m + "dq.norm")), up.vec(st.f32(m + "dkv.norm"))
         else:
             raise ConfigError(f"layer {i}: mixer type {kind!r} is not known")
+        L.form, L.mix_scale = LAYER_SEQUENTIAL, 1.0
         layers.append(L)
     top = dict(width=width, vocab=int(cfg["vocab"]), canon_taps=taps, norm_eps=float(cfg["norm"]["eps"]), norm_offset=1.0,
                logit_scale=float(cfg["logit_scale"]), embed=up.mat(st.bf16_bits("embed")), head=up.mat(st.bf16_bits("head")),
@@ -90,7 +101,100 @@ def _expect(st: SafeTensors, name: str, shape: tuple) -> np.ndarray:
     return st.f32(name)
 
 
-ARCHITECTURES = {"Ranutar": _ranutar_layers}
+def _stack(st: SafeTensors, names: list) -> np.ndarray:
+    return np.concatenate([st.bf16_bits(n) for n in names], axis=0)
+
+
+def window_attention_mixer(L, st: SafeTensors, up, m: str, mc: dict, where: str):
+    """Fill descriptor L with a windowed-attention mixer (MIX_WINATTN) from the tensors under prefix m and its configuration mc.  Whatever the
+    configuration or the file does not have does not exist: no bias, no norm, no temperature, no sink, no gate, no rotation, no pooled blocks."""
+    L.kind = MIX_WINATTN
+    L.heads, L.dim = int(mc["heads"]), int(mc["dim"])
+    L.kv_heads, L.vdim = int(mc.get("kv_heads") or L.heads), int(mc.get("vdim") or L.dim)
+    if L.heads % L.kv_heads:
+        raise ConfigError(f"{where}: {L.heads} heads over {L.kv_heads} key / value heads")
+    mask, rot = mc.get("mask") or {}, mc.get("rot") or {}
+    L.window, L.pool = int(mask.get("size") or 0), int(mask.get("pool") or 0)
+    L.rot_dims, L.rot_base, L.rot_pairing = int(rot.get("dims") or 0), float(rot.get("base") or 10000.0), ROT_NEIGHBOURS
+    L.rot_factor = float((rot.get("scaling") or {}).get("factor") or 1.0)
+    L.scale = float(mc["scale"]) if mc.get("scale") is not None else L.dim ** -0.5
+    rows = [(m + "q", L.heads * L.dim), (m + "k", L.kv_heads * L.dim), (m + "v", L.kv_heads * L.vdim)]
+    L.gated = int(m + "g" in st)
+    if L.gated:
+        rows.append((m + "g", L.heads))
+    for n, r in rows:
+        if st.shape(n)[0] != r:
+            raise ConfigError(f"tensor {n}: {st.shape(n)[0]} rows, the configuration gives {r}")
+    L.in_cat = up.mat(_stack(st, [n for n, _ in rows]))
+    if any(n + ".b" in st for n, _ in rows):
+        L.in_bias = up.vec(np.concatenate([_expect(st, n + ".b", (r,)) if n + ".b" in st else np.zeros(r, np.float32) for n, r in rows]))
+    if m + "q.norm" in st:
+        L.qnorm = up.vec(_expect(st, m + "q.norm", (L.heads * L.dim,)))
+    if m + "k.norm" in st:
+        L.knorm = up.vec(_expect(st, m + "k.norm", (L.kv_heads * L.dim,)))
+    if m + "temp" in st:
+        L.temp = up.vec(_expect(st, m + "temp", (L.heads,)))
+    if m + "sink" in st:
+        L.sink = up.vec(_expect(st, m + "sink", (L.heads,)))
+    L.out = up.mat(st.bf16_bits(m + "o"))
+
+
+def gated_linear_mixer(L, st: SafeTensors, up, m: str, mc: dict, where: str):
+    """Fill descriptor L with a gated-linear-attention mixer (MIX_GLA)."""
+    L.kind = MIX_GLA
+    L.heads, L.dim = int(mc["heads"]), int(mc["dim"])
+    L.vdim, L.tau = int(mc.get("vdim") or L.dim), float(mc.get("tau") or 1.0)
+    L.decay_rank = st.shape(m + "a1")[0]
+    for n, r in (("q", L.heads * L.dim), ("k", L.heads * L.dim), ("v", L.heads * L.vdim), ("g", L.heads * L.vdim)):
+        if st.shape(m + n)[0] != r:
+            raise ConfigError(f"tensor {m + n}: {st.shape(m + n)[0]} rows, the configuration gives {r}")
+    L.in_cat = up.mat(_stack(st, [m + n for n in ("q", "k", "v", "g", "a1")]))
+    L.decay2 = up.mat(st.bf16_bits(m + "a2"))
+    L.decay0 = up.vec(_expect(st, m + "a2.b", (L.heads * L.dim,)) if m + "a2.b" in st else np.zeros(L.heads * L.dim, np.float32))
+    L.onorm = up.vec(_expect(st, m + "norm", (L.vdim,)))
+    L.out = up.mat(st.bf16_bits(m + "o"))
+
+
+def _vobisun_layers(cfg: dict, st: SafeTensors, up) -> tuple[list, dict]:
+    width = int(cfg["width"])
+    taps = int((cfg.get("canon") or {}).get("taps") or 1)
+    layers, keep = [], []
+    for i, lc in enumerate(cfg["layers"]):
+        p, mc, kind = f"l{i}.", lc["mixer"], lc["type"]
+        L = hip.SeqLayer()
+        L.form = LAYER_PARALLEL
+        L.norm1 = up.vec(_expect(st, p + "norm1", (width,)))
+        L.canon1 = up.vec(_expect(st, p + "canon1", (width, taps)) if p + "canon1" in st else np.zeros((width, taps), np.float32))
+        mlp = lc.get("mlp")
+        if mlp:
+            if mlp.get("kind") != "dense":
+                raise ConfigError(f"layer {i}: feed-forward kind {mlp.get('kind')!r} is not known")
+            L.ff_kind, L.ff = FF_DENSE_SWIGLU, int(mlp["ff"])
+            gate, upw = st.bf16_bits(p + "mlp.gate"), st.bf16_bits(p + "mlp.up")
+            if gate.shape != (L.ff, width) or upw.shape != (L.ff, width):
+                raise ConfigError(f"layer {i}: feed-forward shapes {gate.shape} / {upw.shape}, the configuration gives {(L.ff, width)}")
+            L.ff_up = up.mat(np.stack([gate, upw], axis=1).reshape(2 * L.ff, width))  # rows gate_0, up_0, gate_1, ...: the pair meets in one epilogue
+            L.ff_down = up.mat(st.bf16_bits(p + "mlp.down"))
+        if kind == "parallel":
+            window_attention_mixer(L, st, up, p + "mix.left.", mc["left"], f"layer {i} (left)")
+            L.mix_scale = float(mc.get("left_scale", 1.0))
+            R = hip.SeqLayer()
+            gated_linear_mixer(R, st, up, p + "mix.right.", mc["right"], f"layer {i} (right)")
+            R.mix_scale = float(mc.get("right_scale", 1.0))
+            keep.append(R)
+            L.beside = C.pointer(R)
+        else:
+            raise ConfigError(f"layer {i}: mixer type {kind!r} is not known")
+        layers.append(L)
+    loop = cfg.get("loop") or {}
+    top = dict(width=width, vocab=int(cfg["vocab"]), canon_taps=taps, norm_eps=float(cfg["norm"]["eps"]), norm_offset=0.0, logit_scale=1.0,
+               embed_scale=float((cfg.get("embedding") or {}).get("scale") or 1.0), loop_start=int(loop.get("start", 0)), loop_stop=int(loop.get("stop", 0)),
+               loop_times=int(loop.get("times", 1)) if loop else 1, embed=up.mat(st.bf16_bits("embed")), head=up.mat(st.bf16_bits("head")),
+               final_norm=up.vec(_expect(st, "final.norm", (width,))), _keep=keep)
+    return layers, top
+
+
+ARCHITECTURES = {"Ranutar": _ranutar_layers, "Vobisun": _vobisun_layers}
 
 
 def read_config(model_dir: str) -> dict:
@@ -122,7 +226,7 @@ class SeqModel:
     """ps_hip_seq over a model directory.  dtype "bfloat16": matrix products on bfloat16 operands, fp32 accumulation; "float32": fp32
     throughout.  Sequences live in slots (acquire / release); forward() is the step function, generate() the greedy / sampled loop."""
 
-    def __init__(self, ctx: hip.Ctx, model_dir: str, dtype: str = "bfloat16", max_batch: int = 256, n_slots: int = 2):
+    def __init__(self, ctx: hip.Ctx, model_dir: str, dtype: str = "bfloat16", max_batch: int = 256, n_slots: int = 2, max_context: int = 0):
         if dtype not in ("bfloat16", "float32"):
             raise ConfigError(f"dtype {dtype!r}: bfloat16 or float32")
         self.ctx, self.dtype = ctx, dtype
@@ -134,6 +238,8 @@ class SeqModel:
         self._layers = (hip.SeqLayer * len(layers))(*layers)
         d = hip.SeqDesc()
         d.n_layers, d.max_batch, d.n_slots, d.compute = len(layers), int(max_batch), int(n_slots), int(dtype == "float32")
+        d.max_context = int(max_context)  # most tokens of one sequence, for the memory that grows with it (0: the library's default)
+        self._keep = top.pop("_keep", None)  # descriptors of second mixers, pointed to from the layers
         for k, v in top.items():
             setattr(d, k, v)
         d.layers = self._layers
@@ -141,6 +247,7 @@ class SeqModel:
         h = C.c_void_p()
         ctx.check(ctx.L.ps_hip_seq_create(ctx.h, C.byref(d), C.byref(h)))
         self.h = h
+        self.n_runs = int(ctx.L.ps_hip_seq_layer_runs(h))  # executions of a layer per forward (a looped stretch counts every time)
         self._dbg = None
 
     def close(self):
@@ -213,9 +320,9 @@ class SeqModel:
 
     # ---- diagnostics
     def capture_layers(self, on: bool = True):
-        """Keep the residual stream after every layer of the next forwards (each at most max_batch tokens)."""
+        """Keep the residual stream after every layer run of the next forwards (each at most max_batch tokens)."""
         if on and self._dbg is None:
-            self._dbg = self.ctx.empty((self.n_layers, self.max_batch, self.width), np.float32)
+            self._dbg = self.ctx.empty((self.n_runs, self.max_batch, self.width), np.float32)
         self.ctx.check(self.ctx.L.ps_hip_seq_debug_layers(self.h, self._dbg.ptr if on else None))
 
     def layers(self, n_tokens: int) -> np.ndarray:
@@ -234,6 +341,7 @@ def load_model(ctx: hip.Ctx, model_dir: str, **kw):
     if os.path.exists(os.path.join(model_dir, "model.json")):
         kw.pop("dtype", None)
         kw.pop("n_slots", None)
+        kw.pop("max_context", None)
         return hip.Model(ctx, model_dir, **kw)
     raise ConfigError(f"{model_dir}: neither config.json + model.safetensors nor model.json + ggml/weights.gguf")
 

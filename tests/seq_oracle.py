@@ -157,3 +157,134 @@ def run(cfg, W, tokens, per_layer=None, window_override=None):
         if per_layer is not None:
             per_layer.append(x.copy())
     return offset_norm(x, W["final.norm"], eps) @ W["head"].T * cfg["logit_scale"]
+
+
+# ---------------------------------------------------------------------------------------------------------------------------------
+# Vobisun: parallel layers (one norm; mixer and feed-forward read it, only the mixer's copy passes the input filter), a mixer made of two
+# mixers side by side -- windowed attention with pooled blocks behind the window and a sink, and gated linear attention -- a SiLU-gated
+# feed-forward, plain norm weights, a scaled embedding, and a run of layers that is repeated with the same weights.
+
+def plain_norm(a, w, eps):
+    return unit_rms(a, eps) * w
+
+
+def rotate_pairs(vec, pos, base, dims, factor=1.0):
+    """Neighbours (2i, 2i+1), i < dims/2, turn by pos * base^(-2i/dims) / factor; the rest of vec is kept."""
+    out = np.array(vec, dtype=np.float64)
+    for i in range(dims // 2):
+        ang = pos * (base ** (-2.0 * i / dims) / factor)
+        a, b = vec[..., 2 * i], vec[..., 2 * i + 1]
+        out[..., 2 * i] = a * np.cos(ang) - b * np.sin(ang)
+        out[..., 2 * i + 1] = b * np.cos(ang) + a * np.sin(ang)
+    return out
+
+
+def visible_tokens(i, size):
+    """Positions a query at i sees directly."""
+    return range(max(0, i - size + 1), i + 1)
+
+
+def visible_blocks(i, size, pool):
+    """Blocks of `pool` positions that lie wholly before the window of a query at i."""
+    if not pool:
+        return range(0)
+    return range(max(0, (i - size + 1) // pool)) if i - size + 1 > 0 else range(0)
+
+
+def pooled_window_attention(W, pre, h, mc, eps, size=None, pool=None, use_sink=True):
+    """Soft-max attention over the last `size` tokens plus one mean key / value per block of `pool` tokens wholly before them, a sink in
+    the denominator, a per-head temperature, norms over the whole q and k projections, neighbour-pair rotary, a sigmoid gate per head."""
+    T = h.shape[0]
+    H, G, d, dv = mc["heads"], mc["kv_heads"], mc["dim"], mc["vdim"]
+    mask = mc.get("mask") or {}
+    size = (mask.get("size") or T + 1) if size is None else size
+    pool = mask.get("pool", 0) if pool is None else pool
+    rot = mc.get("rot") or {}
+    dims, base = rot.get("dims", 0), rot.get("base", 10000.0)
+    factor = (rot.get("scaling") or {}).get("factor", 1.0)
+
+    def proj(n):
+        y = h @ W[pre + n].T
+        return y + W[pre + n + ".b"] if pre + n + ".b" in W else y
+
+    q, k, v = proj("q"), proj("k"), proj("v").reshape(T, G, dv)
+    if pre + "q.norm" in W:
+        q = plain_norm(q, W[pre + "q.norm"], eps)
+    if pre + "k.norm" in W:
+        k = plain_norm(k, W[pre + "k.norm"], eps)
+    q, k = q.reshape(T, H, d), k.reshape(T, G, d)
+    for t in range(T):
+        q[t], k[t] = rotate_pairs(q[t], t, base, dims, factor), rotate_pairs(k[t], t, base, dims, factor)
+    gate = 1.0 / (1.0 + np.exp(-(h @ W[pre + "g"].T))) if pre + "g" in W else np.ones((T, H))
+    temp = W[pre + "temp"] if pre + "temp" in W else np.ones(H)
+    out = np.zeros((T, H, dv))
+    for t in range(T):
+        toks, blocks = list(visible_tokens(t, size)), list(visible_blocks(t, size, pool))
+        for hd in range(H):
+            g = hd // (H // G)
+            keys = [k[b * pool:(b + 1) * pool, g].mean(axis=0) for b in blocks] + [k[s, g] for s in toks]
+            vals = [v[b * pool:(b + 1) * pool, g].mean(axis=0) for b in blocks] + [v[s, g] for s in toks]
+            sc = np.array([q[t, hd] @ kk for kk in keys]) * mc["scale"] * temp[hd]
+            top = max(sc.max(), W[pre + "sink"][hd]) if use_sink and pre + "sink" in W else sc.max()
+            e = np.exp(sc - top)
+            den = e.sum() + (np.exp(W[pre + "sink"][hd] - top) if use_sink and pre + "sink" in W else 0.0)
+            out[t, hd] = sum(e[n] * vals[n] for n in range(len(keys))) / den * gate[t, hd]
+    return out.reshape(T, H * dv) @ W[pre + "o"].T
+
+
+def gated_linear_attention(W, pre, h, mc, eps):
+    """S <- diag(alpha) S + k v^T,  o = S^T q  per head, alpha = sigmoid(z)^(1/tau) per key channel from a two-matrix projection."""
+    T = h.shape[0]
+    H, d, dv, tau = mc["heads"], mc["dim"], mc["vdim"], mc["tau"]
+    q = (h @ W[pre + "q"].T * d ** -0.5).reshape(T, H, d)
+    k = (h @ W[pre + "k"].T).reshape(T, H, d)
+    v = (h @ W[pre + "v"].T).reshape(T, H, dv)
+    z = (h @ W[pre + "a1"].T) @ W[pre + "a2"].T + W[pre + "a2.b"]
+    alpha = np.exp(-softplus(-z) / tau).reshape(T, H, d)
+    S = np.zeros((H, d, dv))
+    o = np.zeros((T, H, dv))
+    for t in range(T):
+        for hd in range(H):
+            S[hd] = alpha[t, hd][:, None] * S[hd] + np.outer(k[t, hd], v[t, hd])
+            o[t, hd] = S[hd].T @ q[t, hd]
+    o = plain_norm(o, W[pre + "norm"], eps).reshape(T, H * dv) * silu(h @ W[pre + "g"].T)
+    return o @ W[pre + "o"].T
+
+
+def side_by_side_mixer(W, pre, h, mc, eps, **kw):
+    return mc["left_scale"] * pooled_window_attention(W, pre + "left.", h, mc["left"], eps, **kw) + \
+        mc["right_scale"] * gated_linear_attention(W, pre + "right.", h, mc["right"], eps)
+
+
+def gated_feed_forward(W, pre, h):
+    return (silu(h @ W[pre + "gate"].T) * (h @ W[pre + "up"].T)) @ W[pre + "down"].T
+
+
+def layer_runs(cfg):
+    """Indices of the layers in the order they run: the looped stretch `times` times in a row."""
+    n, loop = len(cfg["layers"]), cfg.get("loop")
+    if not loop:
+        return list(range(n))
+    a, b = loop["start"], loop["stop"]
+    return list(range(a)) + list(range(a, b)) * loop["times"] + list(range(b, n))
+
+
+def run_parallel(cfg, W, tokens, per_layer=None, **kw):
+    """Logits [T, vocab] of a whole sequence of the parallel-layer design; kw overrides the attention's size / pool / use_sink on purpose
+    (a WRONG model for sensitivity checks)."""
+    W = {k: np.asarray(v, dtype=np.float64) for k, v in W.items()}
+    eps = cfg["norm"]["eps"]
+    x = W["embed"][np.asarray(tokens)] * (cfg.get("embedding") or {}).get("scale", 1.0)
+    for i in layer_runs(cfg):
+        lc, p = cfg["layers"][i], "l%d." % i
+        h = plain_norm(x, W[p + "norm1"], eps)
+        hm = h + time_conv(h, W[p + "canon1"]) if p + "canon1" in W else h
+        if lc["type"] != "parallel":
+            raise ValueError(lc["type"])
+        y = side_by_side_mixer(W, p + "mix.", hm, lc["mixer"], eps, **kw)
+        if lc.get("mlp"):
+            y = y + gated_feed_forward(W, p + "mlp.", h)
+        x = x + y
+        if per_layer is not None:
+            per_layer.append(x.copy())
+    return plain_norm(x, W["final.norm"], eps) @ W["head"].T
