@@ -157,3 +157,178 @@ void psk_winattn(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int 
     hipLaunchKernelGGL(winattn_kernel, dim3(T, H), dim3(64), (size_t)(d + 64) * 4, st, step, (long long)ring_off, cap, (long long)pool_off, pool, q, (long long)ldq, gate,
                        (long long)ldg, temp, sink, H, G, d, dv, window, scale, o, (long long)ldo);
 }
+
+// ---------------------------------------------------------------------------------------------------- matrix-core forms (ps_attn_dev.h)
+// A portion: block = 64 consecutive tokens of one head (a wave per 16).  The visible block means first (key index = block), then the window's ring rows
+// (key index = position), one online soft-max over both.  dynamic LDS: 4 x (16 x (d + 4) + 16 x 17)
+template <int NJ>
+__global__ __launch_bounds__(256) void winattn_mfma_kernel(const ps_seq_step *step, long long ring_off, int cap, long long pool_off, int pool, const float *q, long long ldq,
+                                                           const float *gate, long long ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window,
+                                                           float scale, int T, float *o, long long ldo) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lq = lane >> 4, h = blockIdx.y, g = h / (H / G);
+    const int qld = d + 4;
+    float *qs = lds + wave * (16 * qld + 16 * 17), *pt = qs + 16 * qld;
+    const long long pos0 = step->pos0;
+    const int t0 = blockIdx.x * 64 + wave * 16;
+    if (t0 >= T) return; // (no block-wide barrier below: waves are on their own)
+    for (int r = 0; r < 16; r++) {
+        const int t = t0 + r;
+        const float *qt = q + (long long)(t < T ? t : 0) * ldq + (long long)h * d;
+        for (int c = lane; c < d; c += 64) qs[r * qld + c] = t < T ? qt[c] : 0.f;
+    }
+    __builtin_amdgcn_wave_barrier();
+    const long long rs = (long long)G * (d + dv);
+    const float *ring = step->state + ring_off, *means = step->state + pool_off;
+    const float sc = scale * (temp ? temp[h] : 1.f);
+    long long rowlo[4], rowhi[4], blo[4], bhi[4];
+    float m[4], l[4];
+    la_f4 acc[NJ];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const long long rp = pos0 + t0 + 4 * lq + i;
+        const bool in = t0 + 4 * lq + i < T;
+        rowlo[i] = in && rp - window + 1 > 0 ? rp - window + 1 : 0;
+        rowhi[i] = in ? rp + 1 : 0;
+        blo[i] = 0;
+        bhi[i] = in ? wa_blocks(rp, window, pool) : 0;
+        m[i] = -INFINITY; l[i] = 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < NJ; j++) acc[j] = la_f4{0.f, 0.f, 0.f, 0.f};
+    const long long plast = pos0 + (t0 + 15 < T ? t0 + 15 : T - 1), pfirst = pos0 + t0;
+    const long long nbmax = wa_blocks(plast, window, pool);
+    {
+        const la_src k1 = {means + (long long)g * d, rs, 0, 0}, vs = {means + (long long)G * d + (long long)g * dv, rs, 0, 0};
+        for (long long j0 = 0; j0 < nbmax; j0 += 16) la_tile<NJ>(qs, qld, pt, k1, k1, vs, d, 0, dv, j0, nbmax, blo, bhi, sc, m, l, acc);
+    }
+    {
+        const la_src k1 = {ring + (long long)g * d, rs, 0, cap}, vs = {ring + (long long)G * d + (long long)g * dv, rs, 0, cap};
+        const long long lo = pfirst - window + 1 > 0 ? pfirst - window + 1 : 0;
+        for (long long j0 = lo; j0 <= plast; j0 += 16) la_tile<NJ>(qs, qld, pt, k1, k1, vs, d, 0, dv, j0, plast + 1, rowlo, rowhi, sc, m, l, acc);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int t = t0 + 4 * lq + i;
+        if (t >= T) continue;
+        const float f = wa_finish(m[i], l[i], sink, h) * (gate ? wa_sigmoid(gate[(long long)t * ldg + h]) : 1.f);
+#pragma unroll
+        for (int J = 0; J < NJ / 4; J++) { // a lane's four tiles of a 64-column group are four consecutive columns: one 16-byte store
+            const int c = 64 * J + 4 * lr;
+            if (c < dv) *(la_f4 *)(o + (long long)t * ldo + (long long)h * dv + c) = la_f4{acc[4 * J][i] * f, acc[4 * J + 1][i] * f, acc[4 * J + 2][i] * f, acc[4 * J + 3][i] * f};
+        }
+    }
+}
+
+static size_t wa_mfma_lds(int d) { return (size_t)4 * (16 * (d + 4) + 16 * 17) * 4; }
+// the sizes the matrix-core forms take: 16-byte pieces of keys (d a multiple of 16) and values (dv of 4, at most 128 columns per head)
+bool psk_winattn_mfma_ok(int d, int dv) { return d % 16 == 0 && dv % 4 == 0 && dv <= 128 && wa_mfma_lds(d) <= 160 * 1024; }
+void psk_winattn_mfma(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *q, int64_t ldq, const float *gate,
+                      int64_t ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window, float scale, int T, float *o, int64_t ldo) {
+    static unsigned long long mask = 0;
+    if (ps_first_on_device(&mask)) (void)hipFuncSetAttribute((const void *)winattn_mfma_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    hipLaunchKernelGGL(winattn_mfma_kernel<8>, dim3((T + 63) / 64, H), dim3(256), wa_mfma_lds(d), st, step, (long long)ring_off, cap, (long long)pool_off, pool, q,
+                       (long long)ldq, gate, (long long)ldg, temp, sink, H, G, d, dv, window, scale, T, o, (long long)ldo);
+}
+
+// A single token.  Rows = the heads that share key / value group g (16 per block); the keys are cut into tiles of 16 in one index space -- tiles
+// 0 .. nbt - 1 the visible block means, then the window from its first position -- and wave w of block (x, head tile, g) takes tile 4 x + w.
+// Partials per (tile, head): [o[dv] unnormalised, m, l, -, -], merged by winattn_merge_kernel, where the sink and the gate come in.
+// dynamic LDS: 16 x (d + 4) + 4 x 16 x 17
+template <int NJ>
+__global__ __launch_bounds__(256) void winattn_step_kernel(const ps_seq_step *step, long long ring_off, int cap, long long pool_off, int pool, const float *q,
+                                                           const float *temp, int H, int G, int d, int dv, int window, float scale, float *part) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lq = lane >> 4, g = blockIdx.z, hpg = H / G, r0 = blockIdx.y * 16;
+    const int qld = d + 4;
+    float *qs = lds, *pt = lds + 16 * qld + wave * 16 * 17;
+    const long long p = step->pos0, lo = p - window + 1 > 0 ? p - window + 1 : 0, nb = wa_blocks(p, window, pool), nbt = (nb + 15) / 16;
+    const long long tile = (long long)blockIdx.x * 4 + wave, ntiles = nbt + (p - lo) / 16 + 1;
+    // the group's 16 queries into LDS, each already times its head's temperature (the scores of a tile then share one scale)
+    for (int r = wave; r < 16; r += 4) {
+        const int hh = r0 + r, h = g * hpg + hh;
+        const float tp = hh < hpg && temp ? temp[h] : 1.f;
+        for (int c = lane; c < d; c += 64) qs[r * qld + c] = hh < hpg ? q[(long long)h * d + c] * tp : 0.f;
+    }
+    __syncthreads();
+    if (tile >= ntiles) return;
+    const long long rs = (long long)G * (d + dv);
+    const float *base = tile < nbt ? step->state + pool_off : step->state + ring_off;
+    const la_src k1 = {base + (long long)g * d, rs, 0, tile < nbt ? 0 : (long long)cap}, vs = {base + (long long)G * d + (long long)g * dv, rs, 0, tile < nbt ? 0 : (long long)cap};
+    const long long j0 = tile < nbt ? tile * 16 : lo + (tile - nbt) * 16, jend = tile < nbt ? nb : p + 1;
+    long long rowlo[4], rowhi[4];
+    float m[4], l[4];
+    la_f4 acc[NJ];
+#pragma unroll
+    for (int i = 0; i < 4; i++) { const bool in = r0 + 4 * lq + i < hpg; rowlo[i] = 0; rowhi[i] = in ? jend : 0; m[i] = -INFINITY; l[i] = 0.f; }
+#pragma unroll
+    for (int j = 0; j < NJ; j++) acc[j] = la_f4{0.f, 0.f, 0.f, 0.f};
+    la_tile<NJ>(qs, qld, pt, k1, k1, vs, d, 0, dv, j0, jend, rowlo, rowhi, scale, m, l, acc);
+    const int dvp = dv + 4;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int hh = r0 + 4 * lq + i;
+        if (hh >= hpg) continue;
+        float *pp = part + (tile * H + g * hpg + hh) * dvp;
+        if (lr == 0) { pp[dv] = m[i]; pp[dv + 1] = l[i]; }
+#pragma unroll
+        for (int J = 0; J < NJ / 4; J++) {
+            const int c = 64 * J + 4 * lr;
+            if (c < dv) *(la_f4 *)(pp + c) = la_f4{acc[4 * J][i], acc[4 * J + 1][i], acc[4 * J + 2][i], acc[4 * J + 3][i]};
+        }
+    }
+}
+// o[h][c] = gate_h * sum_tiles exp(m_t - M) o_t[c] / (sum_tiles exp(m_t - M) l_t + exp(sink_h - M)),  M = max(max_t m_t, sink_h)
+__global__ __launch_bounds__(256) void winattn_merge_kernel(const ps_seq_step *step, const float *part, const float *gate, const float *sink, int pool, int H, int dv,
+                                                            int window, int max_tiles, float *o) {
+    extern __shared__ float wts[]; // [max_tiles] weights exp(m_t - M)
+    __shared__ float red[4];
+    const int h = blockIdx.x, tid = threadIdx.x, dvp = dv + 4;
+    const long long p = step->pos0, lo = p - window + 1 > 0 ? p - window + 1 : 0, nb = wa_blocks(p, window, pool);
+    long long ntl = (nb + 15) / 16 + (p - lo) / 16 + 1;
+    const int nt = (int)(ntl < max_tiles ? ntl : max_tiles);
+    float mx = sink ? sink[h] : -INFINITY;
+    for (int t = tid; t < nt; t += 256) mx = fmaxf(mx, part[((long long)t * H + h) * dvp + dv]);
+    mx = wa_wave_max(mx);
+    if ((tid & 63) == 0) red[tid >> 6] = mx;
+    __syncthreads();
+    const float M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    float ls = 0.f;
+    for (int t = tid; t < nt; t += 256) {
+        const float *pp = part + ((long long)t * H + h) * dvp + dv;
+        const float w = pp[0] == -INFINITY ? 0.f : expf(pp[0] - M);
+        wts[t] = w;
+        ls = fmaf(w, pp[1], ls);
+    }
+    ls = wa_wave_sum(ls);
+    if ((tid & 63) == 0) red[tid >> 6] = ls;
+    __syncthreads();
+    const float L = red[0] + red[1] + red[2] + red[3] + (sink ? expf(sink[h] - M) : 0.f);
+    const float f = (gate ? wa_sigmoid(gate[h]) : 1.f) / L;
+    for (int c = tid; c < dv; c += 256) {
+        float a = 0.f;
+#pragma unroll 8
+        for (int t = 0; t < nt; t++) a = fmaf(wts[t], part[((long long)t * H + h) * dvp + c], a);
+        o[(long long)h * dv + c] = a * f;
+    }
+}
+
+static int wa_max_tiles(int window, int pool, int64_t max_context) {
+    const int64_t nb = pool > 0 ? max_context / pool + 1 : 0;
+    return (int)((nb + 15) / 16 + (window + 15) / 16 + 1); // (a window that does not start on a tile's edge touches one tile more)
+}
+size_t psk_winattn_step_scratch(int H, int dv, int window, int pool, int64_t max_context) {
+    return (size_t)(wa_max_tiles(window, pool, max_context) + 4) * H * (dv + 4) * 4;
+}
+// q [H * d] -> o [H * dv]; gate [H] raw or NULL; scratch from psk_winattn_step_scratch
+void psk_winattn_step(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *q, const float *gate, const float *temp,
+                      const float *sink, int H, int G, int d, int dv, int window, float scale, int64_t max_context, float *scratch, float *o) {
+    const int max_tiles = wa_max_tiles(window, pool, max_context);
+    const size_t lds = (size_t)(16 * (d + 4) + 4 * 16 * 17) * 4;
+    static unsigned long long mask = 0;
+    if (ps_first_on_device(&mask)) (void)hipFuncSetAttribute((const void *)winattn_step_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    const dim3 grid((max_tiles + 3) / 4, (H / G + 15) / 16, G);
+    hipLaunchKernelGGL(winattn_step_kernel<8>, grid, dim3(256), lds, st, step, (long long)ring_off, cap, (long long)pool_off, pool, q, temp, H, G, d, dv, window, scale, scratch);
+    hipLaunchKernelGGL(winattn_merge_kernel, dim3(H), dim3(256), (size_t)grid.x * 4 * 4, st, step, scratch, gate, sink, pool, H, dv, window, (int)grid.x * 4, o);
+}

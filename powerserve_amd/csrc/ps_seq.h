@@ -116,3 +116,11 @@ void psk_winattn_prep(hipStream_t st, const ps_seq_step *step, int64_t ring_off,
 // denominator; gate [T][..] raw (sigmoid here; column h, row stride ldg), temp / sink / gate may be NULL.
 void psk_winattn(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *q, int64_t ldq, const float *gate,
                  int64_t ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window, float scale, int T, float *o, int64_t ldo);
+// The same attention on the fp32 matrix cores for a portion, 16 tokens of a head per wave; _ok: the sizes it takes (d a multiple of 16, dv of 4, dv <= 128).
+bool psk_winattn_mfma_ok(int d, int dv);
+void psk_winattn_mfma(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *q, int64_t ldq, const float *gate,
+                      int64_t ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window, float scale, int T, float *o, int64_t ldo);
+// A single token on the matrix cores: rows = the heads of a key / value group, the keys spread over waves, partials merged in a second launch (same sizes).
+size_t psk_winattn_step_scratch(int H, int dv, int window, int pool, int64_t max_context);
+void psk_winattn_step(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *q, const float *gate, const float *temp,
+                      const float *sink, int H, int G, int d, int dv, int window, float scale, int64_t max_context, float *scratch, float *o);

@@ -45,6 +45,7 @@ struct ps_hip_seq {
     float *x = nullptr, *hn = nullptr, *h = nullptr, *y = nullptr, *t1 = nullptr, *t2 = nullptr, *t3 = nullptr, *t4 = nullptr, *kvx = nullptr, *xn = nullptr,
           *logits = nullptr;
     int32_t *tokens = nullptr, *want = nullptr, *amax = nullptr, *ids = nullptr;
+    float *win_scratch = nullptr; // the windowed attention's single-token partials
     float *abs_scratch = nullptr; // the absorbed single-token attention's folded queries, attended latents and per-tile partials
     void *pack = nullptr; // the wide mat-mul's bfloat16 operand copy
     size_t pack_bytes = 0;
@@ -261,6 +262,12 @@ int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) 
                 ab = std::max(ab, psk_latent_absorbed_scratch(P.d.heads, P.d.kv_rank, P.d.window));
         });
         if (ab) ok = ok && alloc((void **)&m->abs_scratch, ab);
+        size_t wb = 0;
+        mixers([&](LayerPlan &P) {
+            if (P.d.kind == PS_MIX_WINATTN && psk_winattn_mfma_ok(P.d.dim, P.d.vdim))
+                wb = std::max(wb, psk_winattn_step_scratch(P.d.heads, P.d.vdim, P.d.window, P.d.pool, m->max_context));
+        });
+        if (wb) ok = ok && alloc((void **)&m->win_scratch, wb);
     }
     if (desc->compute == 0) { // the wide mat-mul's operand copy: the widest input of any matrix x a portion's rows, or the window's rows x the latent
         int64_t kmax = W, kvrows = 0, kvk = 0;
@@ -399,8 +406,16 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
             psk_winattn_prep(st, m->step, P.off_ring, P.cap, P.off_pool, l.pool, m->t1, P.ncat, l.qnorm, l.knorm, D.norm_eps, (int)H, (int)G, (int)d, (int)dv, l.rot_dims,
                              l.rot_pairing, P.freq, T, m->t2, Hd);
             const float *gate = l.gated ? m->t1 + Hd + G * d + G * dv : nullptr;
-            psk_winattn(st, m->step, P.off_ring, P.cap, P.off_pool, l.pool, m->t2, Hd, gate, P.ncat, l.temp, l.sink, (int)H, (int)G, (int)d, (int)dv, l.window, l.scale, T,
-                        m->t3, Hv);
+            const bool mfma = (m->mode & 2) == 0 && (G * (d + dv)) % 4 == 0 && psk_winattn_mfma_ok((int)d, (int)dv);
+            if (mfma && T == 1 && m->win_scratch)
+                psk_winattn_step(st, m->step, P.off_ring, P.cap, P.off_pool, l.pool, m->t2, gate, l.temp, l.sink, (int)H, (int)G, (int)d, (int)dv, l.window, l.scale,
+                                 m->max_context, m->win_scratch, m->t3);
+            else if (mfma)
+                psk_winattn_mfma(st, m->step, P.off_ring, P.cap, P.off_pool, l.pool, m->t2, Hd, gate, P.ncat, l.temp, l.sink, (int)H, (int)G, (int)d, (int)dv, l.window, l.scale,
+                                 T, m->t3, Hv);
+            else
+                psk_winattn(st, m->step, P.off_ring, P.cap, P.off_pool, l.pool, m->t2, Hd, gate, P.ncat, l.temp, l.sink, (int)H, (int)G, (int)d, (int)dv, l.window, l.scale, T,
+                            m->t3, Hv);
             out_proj(m->t3, Hv);
         } else {
             const int64_t dr = l.rot_dim, rs = l.kv_rank + dr, Hv = H * dv, nq = H * (d + dr);
