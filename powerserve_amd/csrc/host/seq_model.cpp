@@ -1,5 +1,6 @@
 #include "seq_model.hpp"
 
+#include <cmath>
 #include <cstring>
 #include <fcntl.h>
 #include <sys/mman.h>
@@ -183,10 +184,132 @@ void ranutar(const JsonValue &cfg, const SafeTensorsFile &st, SeqUploader &up, s
         layers.push_back(L);
     }
 }
+
+// ---------------------------------------------------------------- Vobisun: parallel layers, two mixers side by side, a looped stretch of layers
+double num_or(const JsonValue &o, const std::string &key, double fallback) {
+    return o.kind == JsonValue::OBJ && o.contains(key) && o.at(key).kind == JsonValue::NUM ? o.at(key).num : fallback;
+}
+const JsonValue *obj_or_null(const JsonValue &o, const std::string &key) {
+    return o.kind == JsonValue::OBJ && o.contains(key) && o.at(key).kind == JsonValue::OBJ ? &o.at(key) : nullptr;
+}
+std::vector<float> expect1(const SafeTensorsFile &st, const std::string &n, int64_t r) {
+    const auto &t = st.at(n);
+    if (t.shape.size() != 1 || t.shape[0] != r) POWERSERVE_ABORT("tensor " + n + ": its shape is not what the configuration gives");
+    return st.f32(n);
+}
+// windowed attention with pooled blocks: whatever the configuration or the file does not have does not exist
+void window_attention_mixer(ps_seq_layer &L, const SafeTensorsFile &st, SeqUploader &up, const std::string &m, const JsonValue &mc) {
+    L.kind = PS_MIX_WINATTN;
+    L.heads = (int32_t)mc.at("heads").num;
+    L.dim = (int32_t)mc.at("dim").num;
+    L.kv_heads = (int32_t)num_or(mc, "kv_heads", L.heads);
+    L.vdim = (int32_t)num_or(mc, "vdim", L.dim);
+    if (L.kv_heads <= 0 || L.heads % L.kv_heads) POWERSERVE_ABORT(m + ": heads must be a multiple of kv_heads");
+    if (const JsonValue *mask = obj_or_null(mc, "mask")) { L.window = (int32_t)num_or(*mask, "size", 0); L.pool = (int32_t)num_or(*mask, "pool", 0); }
+    L.rot_pairing = PS_ROT_NEIGHBOURS;
+    L.rot_base = 10000.f;
+    L.rot_factor = 1.f;
+    if (const JsonValue *rot = obj_or_null(mc, "rot")) {
+        L.rot_dims = (int32_t)num_or(*rot, "dims", 0);
+        L.rot_base = (float)num_or(*rot, "base", 10000.0);
+        if (const JsonValue *sc = obj_or_null(*rot, "scaling")) L.rot_factor = (float)num_or(*sc, "factor", 1.0);
+    }
+    L.scale = (float)num_or(mc, "scale", 1.0 / std::sqrt((double)L.dim));
+    L.gated = st.contains(m + "g") ? 1 : 0;
+    std::vector<std::pair<std::string, int64_t>> rows = {{m + "q", (int64_t)L.heads * L.dim}, {m + "k", (int64_t)L.kv_heads * L.dim}, {m + "v", (int64_t)L.kv_heads * L.vdim}};
+    if (L.gated) rows.push_back({m + "g", L.heads});
+    std::vector<std::string> names;
+    std::vector<float> bias;
+    bool any_bias = false;
+    for (const auto &[n, r] : rows) {
+        if (rows_of(st, n) != r) POWERSERVE_ABORT("tensor " + n + ": its rows are not what the configuration gives");
+        names.push_back(n);
+        if (st.contains(n + ".b")) { auto b = expect1(st, n + ".b", r); bias.insert(bias.end(), b.begin(), b.end()); any_bias = true; }
+        else bias.insert(bias.end(), (size_t)r, 0.f);
+    }
+    L.in_cat = mat_rows(st, up, names);
+    if (any_bias) L.in_bias = up.vec(bias);
+    if (st.contains(m + "q.norm")) L.qnorm = up.vec(expect1(st, m + "q.norm", (int64_t)L.heads * L.dim));
+    if (st.contains(m + "k.norm")) L.knorm = up.vec(expect1(st, m + "k.norm", (int64_t)L.kv_heads * L.dim));
+    if (st.contains(m + "temp")) L.temp = up.vec(expect1(st, m + "temp", L.heads));
+    if (st.contains(m + "sink")) L.sink = up.vec(expect1(st, m + "sink", L.heads));
+    L.out = mat1(st, up, m + "o");
+}
+void gated_linear_mixer(ps_seq_layer &L, const SafeTensorsFile &st, SeqUploader &up, const std::string &m, const JsonValue &mc) {
+    L.kind = PS_MIX_GLA;
+    L.heads = (int32_t)mc.at("heads").num;
+    L.dim = (int32_t)mc.at("dim").num;
+    L.vdim = (int32_t)num_or(mc, "vdim", L.dim);
+    L.tau = (float)num_or(mc, "tau", 1.0);
+    L.decay_rank = (int32_t)rows_of(st, m + "a1");
+    const int64_t Hd = (int64_t)L.heads * L.dim, Hv = (int64_t)L.heads * L.vdim;
+    if (rows_of(st, m + "q") != Hd || rows_of(st, m + "k") != Hd || rows_of(st, m + "v") != Hv || rows_of(st, m + "g") != Hv)
+        POWERSERVE_ABORT(m + ": the projections' rows are not what the configuration gives");
+    L.in_cat = mat_rows(st, up, {m + "q", m + "k", m + "v", m + "g", m + "a1"});
+    L.decay2 = mat1(st, up, m + "a2");
+    L.decay0 = up.vec(st.contains(m + "a2.b") ? expect1(st, m + "a2.b", Hd) : std::vector<float>((size_t)Hd, 0.f));
+    L.onorm = up.vec(expect1(st, m + "norm", L.vdim));
+    L.out = mat1(st, up, m + "o");
+}
+
+void vobisun(const JsonValue &cfg, const SafeTensorsFile &st, SeqUploader &up, std::vector<ps_seq_layer> &layers, ps_seq_desc &d) {
+    d.width = (int32_t)cfg.at("width").num;
+    d.vocab = (int32_t)cfg.at("vocab").num;
+    const JsonValue *canon = obj_or_null(cfg, "canon");
+    d.canon_taps = canon ? (int32_t)num_or(*canon, "taps", 1) : 1;
+    d.norm_eps = (float)cfg.at("norm").at("eps").num;
+    d.norm_offset = 0.0f;
+    d.logit_scale = 1.0f;
+    const JsonValue *emb = obj_or_null(cfg, "embedding");
+    d.embed_scale = emb ? (float)num_or(*emb, "scale", 1.0) : 1.0f;
+    d.loop_times = 1;
+    if (const JsonValue *loop = obj_or_null(cfg, "loop")) {
+        d.loop_start = (int32_t)num_or(*loop, "start", 0);
+        d.loop_stop = (int32_t)num_or(*loop, "stop", 0);
+        d.loop_times = (int32_t)num_or(*loop, "times", 1);
+    }
+    d.embed = mat1(st, up, "embed");
+    d.head = mat1(st, up, "head");
+    d.final_norm = up.vec(expect1(st, "final.norm", d.width));
+    const auto &ls = cfg.at("layers").arr;
+    for (size_t i = 0; i < ls.size(); i++) {
+        const JsonValue &lc = ls[i], &mc = lc.at("mixer");
+        const std::string p = "l" + std::to_string(i) + ".", kind = lc.at("type").str;
+        ps_seq_layer L{};
+        L.form = PS_LAYER_PARALLEL;
+        L.norm1 = up.vec(expect1(st, p + "norm1", d.width));
+        L.canon1 = up.vec(st.contains(p + "canon1") ? expect(st, p + "canon1", d.width, d.canon_taps) : std::vector<float>((size_t)d.width * d.canon_taps, 0.f));
+        if (lc.contains("mlp") && lc.at("mlp").kind == JsonValue::OBJ) {
+            const JsonValue &f = lc.at("mlp");
+            if (f.at("kind").str != "dense") POWERSERVE_ABORT("layer " + std::to_string(i) + ": feed-forward kind " + f.at("kind").str + " is not known");
+            L.ff_kind = PS_FF_DENSE_SWIGLU;
+            L.ff = (int32_t)f.at("ff").num;
+            const auto g = st.bf16_bits(p + "mlp.gate"), u = st.bf16_bits(p + "mlp.up");
+            const size_t W = (size_t)d.width;
+            if (g.size() != (size_t)L.ff * W || u.size() != g.size()) POWERSERVE_ABORT("layer " + std::to_string(i) + ": feed-forward shapes");
+            std::vector<uint16_t> both(2 * g.size()); // rows gate_0, up_0, gate_1, ...: the pair meets in one epilogue
+            for (size_t r = 0; r < (size_t)L.ff; r++) {
+                memcpy(&both[(2 * r) * W], &g[r * W], W * 2);
+                memcpy(&both[(2 * r + 1) * W], &u[r * W], W * 2);
+            }
+            L.ff_up = up.mat(both, 2 * (int64_t)L.ff, d.width);
+            L.ff_down = mat1(st, up, p + "mlp.down");
+        }
+        if (kind != "parallel") POWERSERVE_ABORT("layer " + std::to_string(i) + ": mixer type " + kind + " is not known");
+        window_attention_mixer(L, st, up, p + "mix.left.", mc.at("left"));
+        L.mix_scale = (float)num_or(mc, "left_scale", 1.0);
+        ps_seq_layer R{};
+        gated_linear_mixer(R, st, up, p + "mix.right.", mc.at("right"));
+        R.mix_scale = (float)num_or(mc, "right_scale", 1.0);
+        up.beside.push_back(R);
+        L.beside = &up.beside.back();
+        layers.push_back(L);
+    }
+}
 } // namespace
 
 const std::map<std::string, SeqArchitecture> &seq_architectures() {
-    static const std::map<std::string, SeqArchitecture> reg = {{"Ranutar", ranutar}};
+    static const std::map<std::string, SeqArchitecture> reg = {{"Ranutar", ranutar}, {"Vobisun", vobisun}};
     return reg;
 }
 bool is_seq_model_dir(const std::string &dir) {
@@ -195,7 +318,7 @@ bool is_seq_model_dir(const std::string &dir) {
 }
 
 // ---------------------------------------------------------------- the model
-SeqModel::SeqModel(const std::string &model_dir, const std::string &dtype, int device, size_t max_batch, int n_slots) {
+SeqModel::SeqModel(const std::string &model_dir, const std::string &dtype, int device, size_t max_batch, int n_slots, int max_context) {
     if (dtype != "bfloat16" && dtype != "float32") POWERSERVE_ABORT("dtype " + dtype + ": bfloat16 or float32");
     JsonValue cfg;
     try { cfg = JsonValue::parse_file(model_dir + "/config.json"); } catch (const std::exception &e) { POWERSERVE_ABORT(std::string("config.json: ") + e.what()); }
@@ -204,7 +327,7 @@ SeqModel::SeqModel(const std::string &model_dir, const std::string &dtype, int d
     arch = cfg.at("architecture").str;
     SafeTensorsFile st(model_dir + "/model.safetensors");
     if (ps_hip_create(device, &m_ctx) != 0) POWERSERVE_ABORT("no HIP device: the MI355X backend cannot run (there is no CPU fallback)");
-    m_up = SeqUploader{m_ctx, dtype == "float32", {}, {}};
+    m_up = SeqUploader{m_ctx, dtype == "float32", {}, {}, {}};
     std::vector<ps_seq_layer> layers;
     ps_seq_desc d{};
     try {
@@ -214,6 +337,7 @@ SeqModel::SeqModel(const std::string &model_dir, const std::string &dtype, int d
     d.max_batch = (int32_t)max_batch;
     d.n_slots = n_slots;
     d.compute = dtype == "float32";
+    d.max_context = max_context;
     d.layers = layers.data();
     hip_ok(m_ctx, ps_hip_seq_create(m_ctx, &d, &m_h), "ps_hip_seq_create");
     vocab = (uint32_t)d.vocab; width = (uint32_t)d.width; n_layers = (uint32_t)d.n_layers;
@@ -258,9 +382,9 @@ std::vector<Token> SeqModel::generate(const std::vector<Token> &prompt, int step
     release(slot);
     return out;
 }
-auto load_seq_model(const std::string &model_dir, const std::string &dtype, int device, size_t max_batch, int n_slots) -> std::shared_ptr<SeqModel> {
+auto load_seq_model(const std::string &model_dir, const std::string &dtype, int device, size_t max_batch, int n_slots, int max_context) -> std::shared_ptr<SeqModel> {
     if (!is_seq_model_dir(model_dir)) POWERSERVE_ABORT(model_dir + ": config.json + model.safetensors expected");
-    return std::make_shared<SeqModel>(model_dir, dtype, device, max_batch, n_slots);
+    return std::make_shared<SeqModel>(model_dir, dtype, device, max_batch, n_slots, max_context);
 }
 
 } // namespace powerserve
@@ -272,8 +396,8 @@ void psh_set_error(const char *msg);
 void *psh_sampler_create(const void *cfg);
 void psh_sampler_free(void *s);
 int psh_is_seq_model_dir(const char *dir) { return is_seq_model_dir(dir) ? 1 : 0; }
-void *psh_seq_load(const char *model_dir, const char *dtype, int device, int max_batch, int n_slots) {
-    try { return new std::shared_ptr<SeqModel>(load_seq_model(model_dir, dtype, device, (size_t)max_batch, n_slots)); } catch (const std::exception &e) { psh_set_error(e.what()); return nullptr; }
+void *psh_seq_load(const char *model_dir, const char *dtype, int device, int max_batch, int n_slots, int max_context) {
+    try { return new std::shared_ptr<SeqModel>(load_seq_model(model_dir, dtype, device, (size_t)max_batch, n_slots, max_context)); } catch (const std::exception &e) { psh_set_error(e.what()); return nullptr; }
 }
 void psh_seq_free(void *h) { delete (std::shared_ptr<SeqModel> *)h; }
 uint32_t psh_seq_vocab(void *h) { return (*(std::shared_ptr<SeqModel> *)h)->vocab; }

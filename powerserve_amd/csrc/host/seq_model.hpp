@@ -6,6 +6,7 @@
 #include "sampler.hpp"
 #include "../../../include/ps_hip.h"
 
+#include <deque>
 #include <functional>
 #include <map>
 #include <span>
@@ -42,13 +43,14 @@ struct SeqUploader {
     bool as_f32;
     std::vector<void *> vecs;
     std::vector<ps_dense *> mats;
+    std::deque<ps_seq_layer> beside; // descriptors of second mixers, pointed to from the layers (addresses stay put)
     const float *vec(const std::vector<float> &a);
     const ps_dense *mat(const std::vector<uint16_t> &bits, int64_t rows, int64_t cols);
     void free_all();
 };
 
 struct SeqModel {
-    SeqModel(const std::string &model_dir, const std::string &dtype, int device, size_t max_batch, int n_slots);
+    SeqModel(const std::string &model_dir, const std::string &dtype, int device, size_t max_batch, int n_slots, int max_context = 0);
     ~SeqModel();
     SeqModel(const SeqModel &) = delete;
     int acquire();
@@ -71,6 +73,7 @@ private:
 using SeqArchitecture = std::function<void(const JsonValue &cfg, const SafeTensorsFile &st, SeqUploader &up, std::vector<ps_seq_layer> &layers, ps_seq_desc &d)>;
 const std::map<std::string, SeqArchitecture> &seq_architectures();
 bool is_seq_model_dir(const std::string &model_dir);
-auto load_seq_model(const std::string &model_dir, const std::string &dtype = "bfloat16", int device = 0, size_t max_batch = 256, int n_slots = 2) -> std::shared_ptr<SeqModel>;
+auto load_seq_model(const std::string &model_dir, const std::string &dtype = "bfloat16", int device = 0, size_t max_batch = 256, int n_slots = 2,
+                    int max_context = 0) -> std::shared_ptr<SeqModel>;
 
 } // namespace powerserve

@@ -58,7 +58,7 @@ def lib() -> C.CDLL:
         L.psh_kv_op.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_int64]
         L.psh_is_seq_model_dir.argtypes = [C.c_char_p]
         L.psh_seq_load.restype = C.c_void_p
-        L.psh_seq_load.argtypes = [C.c_char_p, C.c_char_p, C.c_int, C.c_int, C.c_int]
+        L.psh_seq_load.argtypes = [C.c_char_p, C.c_char_p, C.c_int, C.c_int, C.c_int, C.c_int]
         L.psh_seq_free.argtypes = [C.c_void_p]
         L.psh_seq_vocab.restype = C.c_uint32
         L.psh_seq_vocab.argtypes = [C.c_void_p]
@@ -415,9 +415,9 @@ class Workspace:
 class HostSeqModel:
     """load_seq_model(dir) of the C++ facade (csrc/host/seq_model.cpp): a layer-list model from config.json + model.safetensors."""
 
-    def __init__(self, model_dir: str, dtype: str = "bfloat16", device: int = 0, max_batch: int = 256, n_slots: int = 2):
+    def __init__(self, model_dir: str, dtype: str = "bfloat16", device: int = 0, max_batch: int = 256, n_slots: int = 2, max_context: int = 0):
         self.L = lib()
-        self.h = self.L.psh_seq_load(model_dir.encode(), dtype.encode(), device, max_batch, n_slots)
+        self.h = self.L.psh_seq_load(model_dir.encode(), dtype.encode(), device, max_batch, n_slots, max_context)
         if not self.h:
             raise HostError(self.L.psh_last_error().decode())
         self.vocab = int(self.L.psh_seq_vocab(self.h))

@@ -228,9 +228,61 @@ def seq_config(width: int, vocab: int, layers: list, taps: int = 3, eps: float =
             "vocab": int(vocab), "width": int(width)}
 
 
+def parallel_layer(ff: int | None, left: dict, right: dict, left_scale: float = 1.0, right_scale: float = 1.0) -> dict:
+    """One entry of a Vobisun configuration's 'layers': the two mixers side by side and the feed-forward (None: none)."""
+    return {"type": "parallel", "mixer": {"left": dict(left), "left_scale": float(left_scale), "right": dict(right), "right_scale": float(right_scale)},
+            "mlp": {"ff": int(ff), "kind": "dense"} if ff else None}
+
+
+def parallel_config(width: int, vocab: int, layers: list, taps: int = 3, eps: float = 1e-6, embed_scale: float = 1.0, loop: tuple | None = None) -> dict:
+    """loop: (start, stop, times) or None"""
+    cfg = {"architecture": "Vobisun", "canon": {"taps": int(taps)}, "embedding": {"scale": float(embed_scale)}, "layers": layers,
+           "norm": {"eps": float(eps)}, "vocab": int(vocab), "width": int(width)}
+    if loop:
+        cfg["loop"] = {"start": int(loop[0]), "stop": int(loop[1]), "times": int(loop[2])}
+    return cfg
+
+
+def _parallel_tensors(cfg: dict, seed: int, decay_rank: int) -> dict:
+    rng = np.random.default_rng(seed)
+    W, taps = cfg["width"], cfg["canon"]["taps"]
+
+    def lin(n, k, gain=1.0):
+        return rng.standard_normal((n, k), dtype=np.float32) * np.float32(gain / np.sqrt(k))
+
+    def vec(n, std=0.1, mean=0.0):
+        return (rng.standard_normal(n, dtype=np.float32) * np.float32(std) + np.float32(mean)).astype(np.float32)
+
+    t = {"embed": rng.standard_normal((cfg["vocab"], W), dtype=np.float32) / np.float32(cfg["embedding"]["scale"])}
+    for i, lc in enumerate(cfg["layers"]):
+        p = f"l{i}."
+        t[p + "norm1"] = vec(W, 0.2, 1.0)
+        t[p + "canon1"] = (rng.standard_normal((W, taps), dtype=np.float32) * np.float32(0.3)).astype(np.float32)
+        if lc.get("mlp"):
+            ff = lc["mlp"]["ff"]
+            t[p + "mlp.gate"], t[p + "mlp.up"], t[p + "mlp.down"] = lin(ff, W), lin(ff, W), lin(W, ff)
+        a, m = lc["mixer"]["left"], p + "mix.left."
+        H, G, d, dv = a["heads"], a.get("kv_heads", a["heads"]), a["dim"], a.get("vdim", a["dim"])
+        for n, rows in (("q", H * d), ("k", G * d), ("v", G * dv)):
+            t[m + n], t[m + n + ".b"] = lin(rows, W), vec(rows, 0.3)
+        t[m + "q.norm"], t[m + "k.norm"] = vec(H * d, 0.2, 1.0), vec(G * d, 0.2, 1.0)
+        t[m + "temp"], t[m + "sink"] = vec(H, 0.3, 1.2), vec(H, 1.0, 0.5)
+        t[m + "g"], t[m + "o"] = lin(H, W), lin(W, H * dv)
+        r, m = lc["mixer"]["right"], p + "mix.right."
+        H, d, dv = r["heads"], r["dim"], r.get("vdim", r["dim"])
+        t[m + "q"], t[m + "k"], t[m + "v"], t[m + "g"], t[m + "o"] = lin(H * d, W), lin(H * d, W), lin(H * dv, W), lin(H * dv, W), lin(W, H * dv)
+        t[m + "a1"], t[m + "a2"], t[m + "a2.b"] = lin(decay_rank, W), lin(H * d, decay_rank), vec(H * d, 1.0, 2.0)
+        t[m + "norm"] = vec(dv, 0.2, 1.0)
+    t["final.norm"], t["head"] = vec(W, 0.2, 1.0), lin(cfg["vocab"], W)
+    return t
+
+
 def seq_tensors(cfg: dict, seed: int = 0, decay_rank: int = 8) -> dict:
     """Random-init tensors of a layer-list configuration, name -> float32 array already rounded to bfloat16 (what the file will hold)."""
     from .safetensors_io import f32_to_bf16_bits
+    if cfg.get("architecture") == "Vobisun":
+        t = _parallel_tensors(cfg, seed, decay_rank)
+        return {k: (f32_to_bf16_bits(v).astype(np.uint32) << 16).view(np.float32).reshape(v.shape) for k, v in t.items()}
     rng = np.random.default_rng(seed)
     W, taps = cfg["width"], cfg["canon"]["taps"]
     t = {}
