@@ -17,11 +17,23 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 SIZES = {
     "2048x6": dict(width=2048, ff=8192, heads=16, dim=128, q_rank=768, kv_rank=512, rot_dim=64, window=1024, layers=6, llama="llama-1b-dims-2l"),
     "4096x3": dict(width=4096, ff=14336, heads=32, dim=128, q_rank=1536, kv_rank=512, rot_dim=64, window=1024, layers=3, llama="llama-8b-dims-4l"),
+    # Vobisun (parallel layers: windowed attention with pooled blocks beside gated linear attention, SiLU-gated feed-forward) at the same widths, feed-forward
+    # sizes, head counts and numbers of layer RUNS; `beside` names the layer-list model it is measured next to
+    "v2048x6": dict(design="Vobisun", width=2048, ff=8192, heads=16, kv_heads=4, dim=128, window=1024, pool=64, rot_dims=64, lin_heads=16, lin_dim=64, lin_vdim=128,
+                    layers=4, loop=(1, 3, 2), beside="2048x6"),
+    "v4096x3": dict(design="Vobisun", width=4096, ff=14336, heads=32, kv_heads=8, dim=128, window=1024, pool=64, rot_dims=64, lin_heads=32, lin_dim=64, lin_vdim=128,
+                    layers=3, loop=None, beside="4096x3"),
 }
 
 
 def config(z: dict, vocab: int = 4096) -> dict:
     H, d = z["heads"], z["dim"]
+    if z.get("design") == "Vobisun":
+        left = dict(heads=H, kv_heads=z["kv_heads"], dim=d, vdim=d, mask={"size": z["window"], "pool": z["pool"]},
+                    rot={"base": 1e6, "dims": z["rot_dims"], "scaling": {"factor": 4.0}}, scale=float(d ** -0.5))
+        right = dict(heads=z["lin_heads"], dim=z["lin_dim"], vdim=z["lin_vdim"], tau=16.0)
+        return synth.parallel_config(z["width"], vocab, [synth.parallel_layer(z["ff"], left, right, 1.0, 1.0) for _ in range(z["layers"])], taps=4,
+                                     embed_scale=float(z["width"] ** 0.5), loop=z["loop"])
     kinds = {
         "delta": dict(heads=H, kv_heads=max(1, H // 2), dim=d, vdim=d, conv=4),
         "latent_attention": dict(heads=H, dim=d, vdim=d, q_rank=z["q_rank"], kv_rank=z["kv_rank"], rot_dim=z["rot_dim"],
@@ -50,12 +62,13 @@ def _kernel(ctx, m, which, T, reps):
 def run_size(ctx, name: str, prompt_len: int, steps: int, max_batch: int, seed: int = 0, with_llama: bool = True) -> dict:
     z = SIZES[name]
     cfg = config(z)
-    out = {"size": name, "config": {k: v for k, v in z.items() if k != "llama"}, "prompt_len": prompt_len, "decode_steps": steps, "portion": max_batch}
+    out = {"size": name, "config": {k: v for k, v in z.items() if k not in ("llama", "beside")}, "prompt_len": prompt_len, "decode_steps": steps, "portion": max_batch}
     with tempfile.TemporaryDirectory() as d:
         t0 = time.time()
         synth.write_seq_model_dir(d, cfg, seed)
-        m = seqmodel.SeqModel(ctx, d, dtype="bfloat16", max_batch=max_batch, n_slots=1)
+        m = seqmodel.SeqModel(ctx, d, dtype="bfloat16", max_batch=max_batch, n_slots=1, max_context=prompt_len + steps + 64)
         out["make_and_load_s"] = round(time.time() - t0, 1)
+    out["layer_runs"] = m.n_runs
     prompt = np.random.default_rng(1).integers(0, cfg["vocab"], prompt_len).astype(np.int32)
     s = m.acquire()
     m.forward(s, prompt[:max_batch])  # untimed: first use of every kernel
@@ -69,7 +82,6 @@ def run_size(ctx, name: str, prompt_len: int, steps: int, max_batch: int, seed: 
     out["decode_tok_s"] = steps / dec
     out["weight_bytes_per_token"] = m.weight_bytes_per_token
     out["decode_hbm_frac"] = m.weight_bytes_per_token * steps / dec / 1e9 / HBM_PEAK_GBS
-    n_mat = sum((4 * 2 + 2) if lc["type"] == "wkv" else 0 for lc in cfg["layers"])  # (only for the record: flops below count every matrix)
     flops_tok = 2.0 * (m.weight_bytes_per_token / 2 - cfg["vocab"] * cfg["width"])
     out["prefill_mfma_frac"] = flops_tok * (prompt_len - 1) / pre / 1e12 / MFMA_BF16_PEAK_TFLOPS
     us, by, fl = _kernel(ctx, m, 0, 1, 20)
@@ -77,7 +89,9 @@ def run_size(ctx, name: str, prompt_len: int, steps: int, max_batch: int, seed: 
     us, by, fl = _kernel(ctx, m, 0, max_batch, 5)
     out["ff_up_matmul"] = {"tokens": max_batch, "us": us, "TFLOPs": fl / us / 1e6, "mfma_frac": fl / us / 1e6 / MFMA_BF16_PEAK_TFLOPS}
     m.close()
-    if with_llama:
+    if z.get("beside"):  # the closest existing model at equal size, same workload
+        out["beside"] = run_size(ctx, z["beside"], prompt_len, steps, max_batch, seed, with_llama=False)
+    if with_llama and z.get("llama"):
         with tempfile.TemporaryDirectory() as d:
             synth.write_model_dir(d, z["llama"], gguf.Q4_K, n_ctx=prompt_len + steps + 64, seed=seed)
             lm = hip.Model(ctx, d, max_batch=512, n_ctx=prompt_len + steps + 64)

@@ -31,15 +31,23 @@ static __device__ __forceinline__ long long wa_blocks(long long p, int window, i
 }
 
 // y[t] = [ q (H d) | k (G d) | v (G dv) | ... ].  q -> qo[t] normed and rotated; k (normed, rotated) and v -> ring row pos mod cap: [G d | G dv].
-__global__ __launch_bounds__(256) void winattn_prep_kernel(const ps_seq_step *step, long long ring_off, int cap, const float *y, long long ldy, const float *qnorm,
-                                                           const float *knorm, float eps, int H, int G, int d, int dv, int rot_dims, int pairing, const float *freq,
-                                                           float *qo, long long ldq) {
+// A step of ONE token also brings its block's sum up to date here (the thread that wrote a channel adds it: the same sum, in the same order, as
+// winattn_pool_kernel makes for a portion).  dynamic LDS: rot_dims floats (cos | sin of the token's angles, shared by all heads).
+__global__ __launch_bounds__(256) void winattn_prep_kernel(const ps_seq_step *step, long long ring_off, int cap, long long pool_off, int pool, const float *y,
+                                                           long long ldy, const float *qnorm, const float *knorm, float eps, int H, int G, int d, int dv, int rot_dims,
+                                                           int pairing, const float *freq, float *qo, long long ldq) {
+    extern __shared__ float cs[];
     __shared__ float red[8];
     const int t = blockIdx.x, tid = threadIdx.x;
     const long long pos = step->pos0 + t;
-    const int nq = H * d, nk = G * d, nv = G * dv;
+    const int nq = H * d, nk = G * d, nv = G * dv, half = rot_dims / 2;
     const float *qt = y + (long long)t * ldy, *kt = qt + nq, *vt = kt + nk;
     float *ring = step->state + ring_off + (pos % cap) * (long long)(nk + nv);
+    for (int i = tid; i < half; i += 256) {
+        const float ang = (float)pos * freq[i];
+        cs[i] = cosf(ang);
+        cs[half + i] = sinf(ang);
+    }
     float a = 0.f, b = 0.f;
     if (qnorm) for (int i = tid; i < nq; i += 256) a += qt[i] * qt[i];
     if (knorm) for (int i = tid; i < nk; i += 256) b += kt[i] * kt[i];
@@ -49,7 +57,6 @@ __global__ __launch_bounds__(256) void winattn_prep_kernel(const ps_seq_step *st
     __syncthreads();
     const float ia = qnorm ? 1.f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)nq + eps) : 1.f;
     const float ib = knorm ? 1.f / sqrtf((red[4] + red[5] + red[6] + red[7]) / (float)nk + eps) : 1.f;
-    const int half = rot_dims / 2;
     // element i of a projection (c = its index in its head): normed, and where c < rot_dims turned together with its partner
     auto turned = [&](const float *src, const float *w, float inv, int i) {
         const int c = i % d;
@@ -60,12 +67,20 @@ __global__ __launch_bounds__(256) void winattn_prep_kernel(const ps_seq_step *st
         if (pairing == PS_ROT_NEIGHBOURS) { partner = i - c + (c ^ 1); pair = c >> 1; first = !(c & 1); }
         else { first = c < half; partner = first ? i + half : i - half; pair = first ? c : c - half; }
         const float other = src[partner] * inv * (w ? w[partner] : 1.f);
-        const float ang = (float)pos * freq[pair], cs = cosf(ang), sn = sinf(ang);
-        return first ? self * cs - other * sn : self * cs + other * sn;
+        return first ? self * cs[pair] - other * cs[half + pair] : self * cs[pair] + other * cs[half + pair];
+    };
+    // the block of a single token: its sum so far (nothing before the block's first position), the mean once the block is complete
+    const bool own_pool = pool > 0 && gridDim.x == 1;
+    const long long pb = own_pool ? pos / pool : 0;
+    float *mean = step->state + pool_off + pb * (long long)(nk + nv);
+    auto pooled = [&](int c, float v) {
+        if (!own_pool) return;
+        const float sum = (pos == pb * pool ? 0.f : mean[c]) + v;
+        mean[c] = pos == pb * pool + pool - 1 ? sum / (float)pool : sum;
     };
     for (int i = tid; i < nq; i += 256) qo[(long long)t * ldq + i] = turned(qt, qnorm, ia, i);
-    for (int i = tid; i < nk; i += 256) ring[i] = turned(kt, knorm, ib, i);
-    for (int i = tid; i < nv; i += 256) ring[nk + i] = vt[i];
+    for (int i = tid; i < nk; i += 256) { const float v = turned(kt, knorm, ib, i); ring[i] = v; pooled(i, v); }
+    for (int i = tid; i < nv; i += 256) { ring[nk + i] = vt[i]; pooled(nk + i, vt[i]); }
 }
 
 // Block sums of the ring rows this step appended, in position order (so the result does not depend on how the tokens were cut into steps); a
@@ -85,9 +100,9 @@ __global__ __launch_bounds__(256) void winattn_pool_kernel(const ps_seq_step *st
 
 void psk_winattn_prep(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *y, int64_t ldy, const float *qnorm,
                       const float *knorm, float eps, int H, int G, int d, int dv, int rot_dims, int pairing, const float *freq, int T, float *q, int64_t ldq) {
-    hipLaunchKernelGGL(winattn_prep_kernel, dim3(T), dim3(256), 0, st, step, (long long)ring_off, cap, y, (long long)ldy, qnorm, knorm, eps, H, G, d, dv, rot_dims, pairing,
-                       freq, q, (long long)ldq);
-    if (pool > 0) {
+    hipLaunchKernelGGL(winattn_prep_kernel, dim3(T), dim3(256), (size_t)(rot_dims + 2) * 4, st, step, (long long)ring_off, cap, (long long)pool_off, pool, y, (long long)ldy,
+                       qnorm, knorm, eps, H, G, d, dv, rot_dims, pairing, freq, q, (long long)ldq);
+    if (pool > 0 && T > 1) {
         const int rs = G * (d + dv);
         hipLaunchKernelGGL(winattn_pool_kernel, dim3((rs + 255) / 256, (T - 1) / pool + 2), dim3(256), 0, st, step, (long long)ring_off, cap, (long long)pool_off, pool, rs);
     }

@@ -27,6 +27,11 @@ struct LayerPlan { // one layer RUN (and, as `side`, the second mixer of one)
     float *freq = nullptr; // rot_dims / 2 angular frequencies (shared by the runs of a layer)
     float act_p = 0.f, act_q = 0.f;
     int64_t ncat = 0, cqkv = 0;
+    // two mixers side by side whose first step is one stacked projection of the same input: the rows of both are ONE matrix (joint, with joint_bias), its
+    // result has in_ld columns and this mixer's part starts at column in_off (in_ld == 0: the mixer multiplies by its own in_cat)
+    const ps_dense *joint = nullptr;
+    const float *joint_bias = nullptr;
+    int64_t in_ld = 0, in_off = 0;
     std::shared_ptr<LayerPlan> side;
 };
 } // namespace
@@ -56,6 +61,7 @@ struct ps_hip_seq {
     std::map<int, hipGraphExec_t> graphs; // single-token greedy step, per slot
     uint64_t weight_bytes = 0;
     std::vector<void *> owned;
+    std::vector<ps_dense *> joints;
 };
 
 __global__ void seq_set_step_kernel(ps_seq_step *s, long long pos0, int n, int slot, float *state, int token0) {
@@ -250,6 +256,39 @@ int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) 
         if (ok) ok = hipMemcpyAsync(P.freq, f.data(), half * 4, hipMemcpyHostToDevice, c->stream) == hipSuccess && hipStreamSynchronize(c->stream) == hipSuccess;
         freq_of[P.d.out] = P.freq;
     });
+    {
+        // the stacked input projections of two mixers side by side, joined once per layer (its runs share the copy)
+        auto stacked = [](int kind) { return kind == PS_MIX_WINATTN || kind == PS_MIX_GLA || kind == PS_MIX_DELTA; };
+        std::map<int, std::pair<const ps_dense *, const float *>> joint_of;
+        for (auto &P : m->L) {
+            if (!ok || !P.side || !stacked(P.d.kind) || !stacked(P.side->d.kind) || P.d.in_cat->dtype != P.side->d.in_cat->dtype) continue;
+            const ps_dense *a = P.d.in_cat, *b = P.side->d.in_cat;
+            auto it = joint_of.find(P.layer);
+            if (it == joint_of.end()) {
+                const size_t es = a->dtype == PS_BF16 ? 2 : 4, na = (size_t)a->N * a->K * es, nb = (size_t)b->N * b->K * es;
+                auto j = new ps_dense();
+                m->joints.push_back(j);
+                j->dtype = a->dtype; j->N = a->N + b->N; j->K = a->K;
+                ok = ok && alloc(&j->data, na + nb) && hipMemcpyAsync(j->data, a->data, na, hipMemcpyDeviceToDevice, c->stream) == hipSuccess &&
+                     hipMemcpyAsync((char *)j->data + na, b->data, nb, hipMemcpyDeviceToDevice, c->stream) == hipSuccess;
+                float *bias = nullptr;
+                if (ok && (P.d.in_bias || P.side->d.in_bias)) {
+                    ok = alloc((void **)&bias, (size_t)j->N * 4);
+                    if (ok) {
+                        psk_fill(c->stream, bias, 0.f, j->N);
+                        if (P.d.in_bias) ok = ok && hipMemcpyAsync(bias, P.d.in_bias, (size_t)a->N * 4, hipMemcpyDeviceToDevice, c->stream) == hipSuccess;
+                        if (P.side->d.in_bias) ok = ok && hipMemcpyAsync(bias + a->N, P.side->d.in_bias, (size_t)b->N * 4, hipMemcpyDeviceToDevice, c->stream) == hipSuccess;
+                    }
+                }
+                ok = ok && hipStreamSynchronize(c->stream) == hipSuccess;
+                it = joint_of.emplace(P.layer, std::make_pair((const ps_dense *)j, (const float *)bias)).first;
+            }
+            P.joint = it->second.first; P.joint_bias = it->second.second;
+            P.in_ld = P.side->in_ld = a->N + b->N;
+            P.in_off = 0; P.side->in_off = a->N;
+            n1 = std::max(n1, P.in_ld);
+        }
+    }
     ok = ok && alloc((void **)&m->step, sizeof(ps_seq_step)) && alloc((void **)&m->x, B * W * 4) && alloc((void **)&m->hn, B * W * 4) && alloc((void **)&m->h, B * W * 4) &&
          alloc((void **)&m->y, B * W * 4) && alloc((void **)&m->t1, B * std::max<int64_t>(n1, 1) * 4) && alloc((void **)&m->t2, B * std::max<int64_t>(n2, 1) * 4) &&
          alloc((void **)&m->t3, B * std::max<int64_t>(n3, 1) * 4) && alloc((void **)&m->t4, B * std::max<int64_t>(n4, 1) * 4) &&
@@ -293,6 +332,7 @@ void ps_hip_seq_destroy(ps_hip_seq *m) {
     (void)hipStreamSynchronize(m->ctx->stream);
     for (auto &g : m->graphs) (void)hipGraphExecDestroy(g.second);
     for (void *p : m->owned) (void)ps_dev_free(p);
+    for (ps_dense *j : m->joints) delete j; // (their data is in `owned`)
     if (m->ids) (void)ps_dev_free(m->ids);
     delete m;
 }
@@ -354,6 +394,8 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
     auto mixer = [&](const LayerPlan &P, float *into, float out_scale) {
         const ps_seq_layer &l = P.d;
         const int64_t H = l.heads, d = l.dim, dv = l.vdim;
+        float *t1 = m->t1 + P.in_off;                       // this mixer's columns of the (possibly joint) input projection
+        const int64_t ld1 = P.in_ld ? P.in_ld : P.ncat;
         auto out_proj = [&](const float *a, int64_t lda) {
             auto g = mm(l.out, a, lda, into ? into : m->y, W);
             g.alpha = out_scale; g.accum = into ? 1 : 0;
@@ -381,40 +423,42 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
             out_proj(m->t3, Hd);
         } else if (l.kind == PS_MIX_DELTA) {
             const int64_t KHd = (int64_t)l.kv_heads * d, Hv = H * dv;
-            psk_dense(st, mm(l.in_cat, m->h, W, m->t1, P.ncat));
-            psk_causal_conv(st, m->step, P.off_conv, m->t1, P.ncat, l.conv, l.conv_taps, 1, P.cqkv, T, m->t2, P.cqkv);
-            psk_delta_scan(st, m->step, P.off_S, m->t2, m->t2 + KHd, m->t2 + 2 * KHd, m->t1 + P.cqkv + Hv, m->t1 + P.cqkv + Hv + H, P.cqkv, P.ncat, l.a_log, l.dt_bias,
+            if (!P.in_ld) psk_dense(st, mm(l.in_cat, m->h, W, t1, ld1));
+            psk_causal_conv(st, m->step, P.off_conv, t1, ld1, l.conv, l.conv_taps, 1, P.cqkv, T, m->t2, P.cqkv);
+            psk_delta_scan(st, m->step, P.off_S, m->t2, m->t2 + KHd, m->t2 + 2 * KHd, t1 + P.cqkv + Hv, t1 + P.cqkv + Hv + H, P.cqkv, ld1, l.a_log, l.dt_bias,
                            (int)H, l.kv_heads, (int)d, (int)dv, T, m->t3, Hv);
-            psk_headnorm_gate(st, m->t3, Hv, m->t1 + P.cqkv, P.ncat, l.onorm, 0, D.norm_eps, (int)H, (int)dv, T);
+            psk_headnorm_gate(st, m->t3, Hv, t1 + P.cqkv, ld1, l.onorm, 0, D.norm_eps, (int)H, (int)dv, T);
             out_proj(m->t3, Hv);
         } else if (l.kind == PS_MIX_GLA) {
             // t1 = [ q | k | v | g | a1 ]; the decay's second matrix (with its bias) -> t2; scan -> t3; per-head norm and gate; out
             const int64_t Hd = H * d, Hv = H * dv;
-            psk_dense(st, mm(l.in_cat, m->h, W, m->t1, P.ncat));
-            auto g2 = mm(l.decay2, m->t1 + 2 * Hd + 2 * Hv, P.ncat, m->t2, Hd);
+            if (!P.in_ld) psk_dense(st, mm(l.in_cat, m->h, W, t1, ld1));
+            auto g2 = mm(l.decay2, t1 + 2 * Hd + 2 * Hv, ld1, m->t2, Hd);
             g2.bias = l.decay0;
             psk_dense(st, g2);
-            psk_gla_scan(st, m->step, P.off_S, m->t1, m->t1 + Hd, m->t1 + 2 * Hd, P.ncat, m->t2, Hd, l.tau, (int)H, (int)d, (int)dv, T, m->t3, Hv);
-            psk_headnorm_gate(st, m->t3, Hv, m->t1 + 2 * Hd + Hv, P.ncat, l.onorm, 0, D.norm_eps, (int)H, (int)dv, T);
+            psk_gla_scan(st, m->step, P.off_S, t1, t1 + Hd, t1 + 2 * Hd, ld1, m->t2, Hd, l.tau, (int)H, (int)d, (int)dv, T, m->t3, Hv);
+            psk_headnorm_gate(st, m->t3, Hv, t1 + 2 * Hd + Hv, ld1, l.onorm, 0, D.norm_eps, (int)H, (int)dv, T);
             out_proj(m->t3, Hv);
         } else if (l.kind == PS_MIX_WINATTN) {
             // t1 = [ q | k | v | gate ] (+ bias); norms, rotation, ring append and block means; attention -> t3; out
             const int64_t G = l.kv_heads, Hd = H * d, Hv = H * dv;
-            auto g = mm(l.in_cat, m->h, W, m->t1, P.ncat);
-            g.bias = l.in_bias;
-            psk_dense(st, g);
-            psk_winattn_prep(st, m->step, P.off_ring, P.cap, P.off_pool, l.pool, m->t1, P.ncat, l.qnorm, l.knorm, D.norm_eps, (int)H, (int)G, (int)d, (int)dv, l.rot_dims,
+            if (!P.in_ld) {
+                auto g = mm(l.in_cat, m->h, W, t1, ld1);
+                g.bias = l.in_bias;
+                psk_dense(st, g);
+            }
+            psk_winattn_prep(st, m->step, P.off_ring, P.cap, P.off_pool, l.pool, t1, ld1, l.qnorm, l.knorm, D.norm_eps, (int)H, (int)G, (int)d, (int)dv, l.rot_dims,
                              l.rot_pairing, P.freq, T, m->t2, Hd);
-            const float *gate = l.gated ? m->t1 + Hd + G * d + G * dv : nullptr;
+            const float *gate = l.gated ? t1 + Hd + G * d + G * dv : nullptr;
             const bool mfma = (m->mode & 2) == 0 && (G * (d + dv)) % 4 == 0 && psk_winattn_mfma_ok((int)d, (int)dv);
             if (mfma && T == 1 && m->win_scratch)
                 psk_winattn_step(st, m->step, P.off_ring, P.cap, P.off_pool, l.pool, m->t2, gate, l.temp, l.sink, (int)H, (int)G, (int)d, (int)dv, l.window, l.scale,
                                  m->max_context, m->win_scratch, m->t3);
             else if (mfma)
-                psk_winattn_mfma(st, m->step, P.off_ring, P.cap, P.off_pool, l.pool, m->t2, Hd, gate, P.ncat, l.temp, l.sink, (int)H, (int)G, (int)d, (int)dv, l.window, l.scale,
+                psk_winattn_mfma(st, m->step, P.off_ring, P.cap, P.off_pool, l.pool, m->t2, Hd, gate, ld1, l.temp, l.sink, (int)H, (int)G, (int)d, (int)dv, l.window, l.scale,
                                  T, m->t3, Hv);
             else
-                psk_winattn(st, m->step, P.off_ring, P.cap, P.off_pool, l.pool, m->t2, Hd, gate, P.ncat, l.temp, l.sink, (int)H, (int)G, (int)d, (int)dv, l.window, l.scale, T,
+                psk_winattn(st, m->step, P.off_ring, P.cap, P.off_pool, l.pool, m->t2, Hd, gate, ld1, l.temp, l.sink, (int)H, (int)G, (int)d, (int)dv, l.window, l.scale, T,
                             m->t3, Hv);
             out_proj(m->t3, Hv);
         } else {
@@ -443,6 +487,12 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
             out_proj(m->t3, Hv);
         }
     };
+    auto joint_in = [&](const LayerPlan &P) { // both mixers' stacked input projections in one product
+        if (!P.joint) return;
+        auto g = mm(P.joint, m->h, W, m->t1, P.in_ld);
+        g.bias = P.joint_bias;
+        psk_dense(st, g);
+    };
     auto ff_up = [&](const LayerPlan &P, const float *in) {
         const ps_seq_layer &l = P.d;
         auto g = mm(l.ff_up, in, W, m->t4, l.ff);
@@ -459,6 +509,7 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
         if (l.form == PS_LAYER_PARALLEL) {
             // hn = norm(x), h = conv(hn); both mixers and the feed-forward add their output projections straight into the residual stream
             boundary(nullptr, nullptr, l.norm1, l.canon1, P.off_canon1);
+            joint_in(P);
             mixer(P, m->x, l.mix_scale);
             if (P.side) mixer(*P.side, m->x, P.side->d.mix_scale);
             if (l.ff_kind != PS_FF_NONE) {
@@ -470,6 +521,7 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
         } else {
             const bool summed = P.side != nullptr || l.mix_scale != 1.f;
             if (summed) psk_fill(st, m->y, 0.f, (int64_t)T * W);
+            joint_in(P);
             mixer(P, summed ? m->y : nullptr, l.mix_scale);
             if (P.side) mixer(*P.side, m->y, P.side->d.mix_scale);
             const bool nseq = next && next->d.form == PS_LAYER_SEQUENTIAL;

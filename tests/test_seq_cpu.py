@@ -86,13 +86,16 @@ def test_unknown_names_are_refused(tmp_path):
 
 def test_ctypes_descriptors_match_the_header(tmp_path):
     src = tmp_path / "sz.c"
-    src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "ps_hip.h"\nint main(void){printf("%zu %zu %zu %zu %zu %zu\\n", sizeof(ps_seq_layer), '
-                   'offsetof(ps_seq_layer, norm1), offsetof(ps_seq_layer, kvnorm), sizeof(ps_seq_desc), offsetof(ps_seq_desc, embed), offsetof(ps_seq_desc, layers));return 0;}\n')
+    src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "ps_hip.h"\nint main(void){printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu\\n", sizeof(ps_seq_layer), '
+                   'offsetof(ps_seq_layer, norm1), offsetof(ps_seq_layer, kvnorm), sizeof(ps_seq_desc), offsetof(ps_seq_desc, embed), offsetof(ps_seq_desc, layers), '
+                   'offsetof(ps_seq_layer, beside), offsetof(ps_seq_layer, in_bias), offsetof(ps_seq_layer, tau), offsetof(ps_seq_desc, embed_scale), '
+                   'offsetof(ps_seq_desc, max_context));return 0;}\n')
     exe = str(tmp_path / "sz")
     subprocess.run(["gcc", "-I" + os.path.join(ROOT, "include"), str(src), "-o", exe], check=True)
     got = [int(x) for x in subprocess.run([exe], check=True, capture_output=True, text=True).stdout.split()]
     assert got == [C.sizeof(hip.SeqLayer), hip.SeqLayer.norm1.offset, hip.SeqLayer.kvnorm.offset, C.sizeof(hip.SeqDesc), hip.SeqDesc.embed.offset,
-                   hip.SeqDesc.layers.offset]
+                   hip.SeqDesc.layers.offset, hip.SeqLayer.beside.offset, hip.SeqLayer.in_bias.offset, hip.SeqLayer.tau.offset, hip.SeqDesc.embed_scale.offset,
+                   hip.SeqDesc.max_context.offset]
 
 
 def test_plain_statement_is_causal_and_windowed():
@@ -109,6 +112,72 @@ def test_plain_statement_is_causal_and_windowed():
     la, lb = seq_oracle.run(only, t2, a), seq_oracle.run(only, t2, b)
     # window 5 and a 2-tap input filter in front of the mixer and of the feed-forward: token 12 reaches positions 12 .. 12 + 4 + 1 + 1
     assert np.abs(la[19:] - lb[19:]).max() < 1e-12 and np.abs(la[12:19] - lb[12:19]).max() > 1e-6
+
+
+PCFG = synth.parallel_config(24, 30, [
+    synth.parallel_layer(20, dict(heads=4, kv_heads=2, dim=6, vdim=10, mask={"size": 5, "pool": 3}, rot={"base": 77.0, "dims": 4, "scaling": {"factor": 2.0}}, scale=0.25),
+                         dict(heads=3, dim=8, vdim=4, tau=5.0), 1.25, 0.5),
+    synth.parallel_layer(None, dict(heads=2, kv_heads=2, dim=6, vdim=6, mask={"size": 4, "pool": 2}, rot={"base": 9.0, "dims": 6}, scale=0.5),
+                         dict(heads=1, dim=5, vdim=7, tau=1.0))], taps=2, eps=1e-5, embed_scale=3.0, loop=(0, 1, 2))
+
+
+def test_parallel_configuration_maps_onto_layer_descriptors(tmp_path):
+    t = synth.write_seq_model_dir(str(tmp_path), PCFG, 1)
+    cfg = seqmodel.read_config(str(tmp_path))
+    up = FakeUp()
+    layers, top = seqmodel.ARCHITECTURES[cfg["architecture"]](cfg, safetensors_io.SafeTensors(str(tmp_path / "model.safetensors")), up)
+    assert (top["width"], top["vocab"], top["canon_taps"], top["norm_offset"], top["embed_scale"]) == (24, 30, 2, 0.0, 3.0)
+    assert (top["loop_start"], top["loop_stop"], top["loop_times"]) == (0, 1, 2)
+    a, b = layers
+    assert (a.form, a.kind, a.heads, a.kv_heads, a.dim, a.vdim, a.window, a.pool, a.rot_dims, a.rot_pairing, a.gated) == \
+        (seqmodel.LAYER_PARALLEL, seqmodel.MIX_WINATTN, 4, 2, 6, 10, 5, 3, 4, seqmodel.ROT_NEIGHBOURS, 1)
+    assert abs(a.rot_base - 77.0) < 1e-6 and a.rot_factor == 2.0 and a.scale == 0.25 and a.mix_scale == 1.25 and b.rot_factor == 1.0
+    r = a.beside.contents
+    assert (r.kind, r.heads, r.dim, r.vdim, r.decay_rank, r.tau, r.mix_scale) == (seqmodel.MIX_GLA, 3, 8, 4, 8, 5.0, 0.5)
+    assert (a.ff_kind, a.ff, b.ff_kind) == (seqmodel.FF_DENSE_SWIGLU, 20, seqmodel.FF_NONE)
+    # stacked input projections: q | k | v | gate with their biases (the gate has none), and q | k | v | g | a1
+    cat = up.mats[a.in_cat - 1001]
+    assert cat.shape == (4 * 6 + 2 * 6 + 2 * 10 + 4, 24)
+    assert np.array_equal(cat, np.concatenate([safetensors_io.f32_to_bf16_bits(t["l0.mix.left." + n]) for n in ("q", "k", "v", "g")]))
+    bias = up.vecs[a.in_bias - 1]
+    assert bias.shape == (60,) and np.array_equal(bias[:24], t["l0.mix.left.q.b"]) and not bias[56:].any()
+    assert up.mats[r.in_cat - 1001].shape == (2 * 3 * 8 + 2 * 3 * 4 + 8, 24)
+    # the feed-forward's gate and up rows alternate
+    both = up.mats[a.ff_up - 1001]
+    assert both.shape == (40, 24)
+    assert np.array_equal(both[0::2], safetensors_io.f32_to_bf16_bits(t["l0.mlp.gate"])) and np.array_equal(both[1::2], safetensors_io.f32_to_bf16_bits(t["l0.mlp.up"]))
+    # what the file does not have does not exist
+    st = safetensors_io.SafeTensors(str(tmp_path / "model.safetensors"))
+    less = {n: st.f32(n) for n in st.names() if not n.endswith((".b", "temp", "sink", "q.norm", "left.g"))}
+    cfg2 = json.loads(json.dumps(PCFG))
+    del cfg2["loop"], cfg2["layers"][0]["mixer"]["left"]["rot"]
+    synth.write_seq_model_dir(str(tmp_path / "less"), cfg2, 1, tensors=less)
+    layers, top = seqmodel.ARCHITECTURES["Vobisun"](cfg2, safetensors_io.SafeTensors(str(tmp_path / "less" / "model.safetensors")), FakeUp())
+    a = layers[0]
+    assert (a.gated, a.in_bias, a.temp, a.sink, a.qnorm, a.rot_dims, top["loop_times"]) == (0, None, None, None, None, 0, 1) and a.knorm is not None
+    bad = json.loads(json.dumps(PCFG))
+    bad["layers"][0]["mixer"]["left"]["heads"] = 5
+    with pytest.raises(seqmodel.ConfigError):
+        seqmodel.ARCHITECTURES["Vobisun"](bad, st, FakeUp())
+
+
+def test_plain_parallel_statement_reach():
+    """causal; with the recurrent mixer switched off, a token reaches exactly as far as its window, then only through its block's mean; the layers of a loop run in order"""
+    assert seq_oracle.layer_runs(PCFG) == [0, 0, 1] and seq_oracle.layer_runs({"layers": [0, 0, 0, 0], "loop": {"start": 1, "stop": 3, "times": 3}}) == [0, 1, 2, 1, 2, 1, 2, 3]
+    assert list(seq_oracle.visible_tokens(9, 4)) == [6, 7, 8, 9] and list(seq_oracle.visible_blocks(9, 4, 3)) == [0, 1] and list(seq_oracle.visible_blocks(8, 4, 3)) == [0]
+    assert list(seq_oracle.visible_blocks(3, 4, 3)) == [] and list(seq_oracle.visible_tokens(2, 4)) == [0, 1, 2]
+    one = synth.parallel_config(24, 30, [synth.parallel_layer(None, PCFG["layers"][0]["mixer"]["left"], PCFG["layers"][0]["mixer"]["right"], 1.0, 0.0)], taps=1)
+    t = synth.seq_tensors(one, 2)
+    rng = np.random.default_rng(0)
+    a = rng.integers(0, 30, 24)
+    b = a.copy()
+    b[7] = (b[7] + 1) % 30
+    la, lb = seq_oracle.run_parallel(one, t, a), seq_oracle.run_parallel(one, t, b)
+    changed = [i for i in range(24) if np.abs(la[i] - lb[i]).max() > 1e-9]
+    # window 5: positions 7 .. 11 see token 7 itself; its block 6 .. 8 is seen from 8 + 5 = 13 on; 12 sees neither
+    assert changed == [7, 8, 9, 10, 11] + list(range(13, 24))
+    la, lb = seq_oracle.run_parallel(one, t, a, pool=0), seq_oracle.run_parallel(one, t, b, pool=0)
+    assert [i for i in range(24) if np.abs(la[i] - lb[i]).max() > 1e-9] == [7, 8, 9, 10, 11]
 
 
 def test_the_small_library_exports_what_its_models_need():
