@@ -4,7 +4,7 @@
 // denominator, a per-head temperature multiplies the scores, a per-head sigmoid gate the output.  What a sequence keeps: a RING of the last
 // `cap` tokens' keys and values (row = position mod cap; cap >= window - 1 + the widest step) and the block means, one row per block, which
 // grow with the sequence.  Scores, soft-max and the weighted sums are fp32.
-//   winattn_prep_kernel    norms over the whole q / k projections, rotation, ring append            (one block per token)
+//   winattn_prep_kernel    norms over the whole q / k projections, rotation, ring append            (one or a few blocks per token)
 //   winattn_pool_kernel    block sums in position order, turned into means when a block is complete  (a thread per channel and block)
 //   winattn_kernel         one wave per (token, head) over [visible blocks | window]: the plain form, any size
 //   winattn_mfma_kernel    a portion on the fp32 matrix cores, 16 tokens of a head per wave (ps_attn_dev.h)
@@ -12,6 +12,7 @@
 #include "ps_attn_dev.h"
 #include "ps_seq.h"
 
+#include <algorithm>
 #include <cmath>
 
 static __device__ __forceinline__ float wa_wave_sum(float v) {
@@ -78,9 +79,17 @@ __global__ __launch_bounds__(256) void winattn_prep_kernel(const ps_seq_step *st
         const float sum = (pos == pb * pool ? 0.f : mean[c]) + v;
         mean[c] = pos == pb * pool + pool - 1 ? sum / (float)pool : sum;
     };
-    for (int i = tid; i < nq; i += 256) qo[(long long)t * ldq + i] = turned(qt, qnorm, ia, i);
-    for (int i = tid; i < nk; i += 256) { const float v = turned(kt, knorm, ib, i); ring[i] = v; pooled(i, v); }
-    for (int i = tid; i < nv; i += 256) { ring[nk + i] = vt[i]; pooled(nk + i, vt[i]); }
+    // the elements of q | k | v are spread over the blocks of a token (gridDim.y; every block has made the sums above for itself)
+    for (int e = blockIdx.y * 256 + tid; e < nq + nk + nv; e += 256 * gridDim.y) {
+        if (e < nq) {
+            qo[(long long)t * ldq + e] = turned(qt, qnorm, ia, e);
+        } else {
+            const int i = e - nq;
+            const float v = i < nk ? turned(kt, knorm, ib, i) : vt[i - nk];
+            ring[i] = v;
+            pooled(i, v);
+        }
+    }
 }
 
 // Block sums of the ring rows this step appended, in position order (so the result does not depend on how the tokens were cut into steps); a
@@ -100,7 +109,9 @@ __global__ __launch_bounds__(256) void winattn_pool_kernel(const ps_seq_step *st
 
 void psk_winattn_prep(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *y, int64_t ldy, const float *qnorm,
                       const float *knorm, float eps, int H, int G, int d, int dv, int rot_dims, int pairing, const float *freq, int T, float *q, int64_t ldq) {
-    hipLaunchKernelGGL(winattn_prep_kernel, dim3(T), dim3(256), (size_t)(rot_dims + 2) * 4, st, step, (long long)ring_off, cap, (long long)pool_off, pool, y, (long long)ldy,
+    const int total = H * d + G * (d + dv);
+    const int split = T >= 64 ? 1 : std::min(16, (total + 511) / 512); // few tokens: a token's elements over several blocks
+    hipLaunchKernelGGL(winattn_prep_kernel, dim3(T, split), dim3(256), (size_t)(rot_dims + 2) * 4, st, step, (long long)ring_off, cap, (long long)pool_off, pool, y, (long long)ldy,
                        qnorm, knorm, eps, H, G, d, dv, rot_dims, pairing, freq, q, (long long)ldq);
     if (pool > 0 && T > 1) {
         const int rs = G * (d + dv);
